@@ -1,6 +1,6 @@
 /*
  * msgl_mix.h -- C ABI of the sequence-mixing kernels (latent attention, linear-recurrence layers, routed experts)
- * for gfx950; implemented by libmsgl_mix.so (mini-sglang_amd/csrc/seqmix.hip, mix_delta.hip).
+ * for gfx950; implemented by libmsgl_mix.so (mini-sglang_amd/csrc/seqmix.hip, mix_delta.hip, mix_par.hip).
  *
  * Same conventions as msgl_hip.h: raw device pointers, explicit sizes and strides in ELEMENTS, `stream` is a
  * hipStream_t passed as void*, every function returns 0 or a negative code and leaves a message for
@@ -27,7 +27,7 @@ extern "C" {
 #define MSGL_MIX_ACT_NONE 0
 #define MSGL_MIX_ACT_RELU2 1 /* max(z, 0)^2 */
 
-#define MSGL_MIX_ABI_VERSION 2
+#define MSGL_MIX_ABI_VERSION 3
 
 const char* msgl_mix_last_error(void);
 int msgl_mix_abi_version(void);
@@ -46,10 +46,11 @@ int msgl_mix_postnorm(const float* x_in, float* x_out, void* h_out, const void* 
 /* One projection row per token = [q: H x (d + r) | latent R | shared rotated key part r] (the last two only with has_kv).
  * Writes the rotated query parts into q_abs[t, h, R : R + r] (fp32, rows of R + r) and, with has_kv, the RMS-normed latent
  * (plain weight c_norm_w) and the rotated key part into cache[out_loc[t]] (rows of R + r, T).
- * cos_sin: fp32 [positions, rot_dims] = cos | sin halves; entries rot_dims .. r of a rotated part pass unchanged. */
+ * cos_sin: fp32 [positions, rot_dims] = cos | sin halves; entries rot_dims .. r of a rotated part pass unchanged.  Pair i of a
+ * rotated part is (i, i + rot_dims / 2), or (2i, 2i + 1) with interleaved != 0. */
 int msgl_mix_latent_prep(const void* proj, int64_t ld_proj, float* q_abs, void* cache, const int* out_loc, const int* positions,
                          const float* cos_sin, const void* c_norm_w, float eps, int tokens, int H, int d, int r, int rot_dims, int R,
-                         int has_kv, int dtype, void* stream);
+                         int has_kv, int interleaved, int dtype, void* stream);
 
 /* Causal attention of H heads over ONE shared key row per token: score = q_abs[t, h] . cache[slot] * scale over dk entries,
  * softmax in fp32, out[t, h] = sum_j p_j cache[slot_j][0 : dv] (fp32).  Requests as in the paged backend: table rows of token
@@ -58,11 +59,12 @@ int msgl_mix_latent_prep(const void* proj, int64_t ld_proj, float* q_abs, void* 
  * bf16 caches run on the matrix cores (Q and the softmax weights rounded to bf16 for the two products, fp32 accumulation and fp32
  * softmax); `splits` > 1 cuts every request's keys into that many ranges whose partial results (workspace: fp32,
  * msgl_mix_latent_attn_workspace_floats) a second launch merges -- for steps with few query rows and many keys.  fp32 caches
- * take the plain fp32 kernel (splits is ignored). */
+ * take the plain fp32 kernel (splits is ignored).
+ * sink (fp32 [H], may be null): one more term exp(sink[h]) in head h's softmax denominator, with no key and no value. */
 int msgl_mix_latent_attn_workspace_floats(int total_q, int H, int dv, int splits);
 int msgl_mix_latent_attn(float* out, const float* q_abs, const void* cache, const int* table, int64_t table_stride, const int* req_rows,
-                         const int* seq_lens, const int* cu_q, int batch, int total_q, int H, int dk, int dv, float scale, int dtype,
-                         int splits, float* workspace, void* stream);
+                         const int* seq_lens, const int* cu_q, int batch, int total_q, int H, int dk, int dv, float scale,
+                         const float* sink, int dtype, int splits, float* workspace, void* stream);
 
 /* Linear recurrence per (request, head): S <- decay[h] S + k v^T, out = S^T q, with q, k, v = SiLU of the projection row
  * [q: H x d | k: H x d | v: H x dv | ...].  state: fp32 [slots, H, d, dv], row slots[b]; a request whose first new token is at
@@ -138,14 +140,15 @@ int msgl_mix_window_attn(void* out, const void* src, int64_t ld_src, int g_off, 
                          int G, int d, int dv, int window, float scale, const float* talk, int dtype, int splits, float* workspace,
                          void* stream);
 
-/* Causal convolution over time per channel, then SiLU: out[t, c] = silu(sum_j taps[c, j] in[pos - (n - 1) + j, c]) (fp32);
+/* Causal convolution over time per channel, then SiLU: out[t, c] = silu(bias[c] + sum_j taps[c, j] in[pos - (n - 1) + j, c]) (fp32;
+ * bias in T, may be null);
  * inputs of this forward are src[t, 0 : C], earlier ones come from state[slots[b]] ([n - 1, C] in T per request: the inputs
  * of the n - 1 positions before the portion), positions before 0 count as zero.  The first `unit_heads` groups of d channels
  * leave as unit vectors (x / sqrt(sum x^2 + 1e-6)), the first `scaled_heads` of them times d^-1/2.  A second launch moves every
  * request's state on to its last n - 1 inputs. */
-int msgl_mix_short_conv(float* out, const void* src, int64_t ld_src, const void* taps, void* state, const int* cu_q, const int* seq_lens,
-                        const int* slots, int batch, int total, int C, int n, int unit_heads, int scaled_heads, int d, int dtype,
-                        void* stream);
+int msgl_mix_short_conv(float* out, const void* src, int64_t ld_src, const void* taps, const void* bias, void* state, const int* cu_q,
+                        const int* seq_lens, const int* slots, int batch, int total, int C, int n, int unit_heads, int scaled_heads, int d,
+                        int dtype, void* stream);
 
 /* Gated delta rule per (request, head): S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  qkv: fp32 rows
  * [q: G x d | k: G x d | v: H x dv] (head h reads q/k group h / (H / G)); state: fp32 [slots, H, d, dv], row slots[b], zero for a
@@ -164,6 +167,64 @@ int msgl_mix_delta_rule(float* out, const float* qkv, float* state, const void* 
 /* out[t, h, e] = o[t, h, e] / sqrt(mean_e(o[t, h]^2) + eps) * w[e] * act(gate[t, h * dv + e]); act: 0 = sigmoid, 1 = SiLU. */
 int msgl_mix_head_gated_norm(void* out, const float* o, const void* gate, int64_t ld_gate, const void* w, float eps, int rows, int H,
                              int dv, int gate_act, int dtype, void* stream);
+
+/* ---- parallel-residual hybrid decoders: token shift, latent attention with a sink, sigmoid attention beside a state-space layer ---- */
+
+/* x32[t] = scale * table[ids[t]] + pair[r]  (fp32).  pair (T, [buckets + 1, W], may be null): r = (previous id * mul_prev + id *
+ * mul_cur) mod buckets, r = buckets for a token at position 0; the id before a portion's first token is prev_tok[req_rows[b]]. */
+int msgl_mix_embed_scaled(float* x32, const void* table, const void* pair, const int* ids, const int* positions, const int* cu_q,
+                          const int* req_rows, int batch, const int* prev_tok, float scale, int buckets, int mul_prev, int mul_cur,
+                          int tokens, int W, int dtype, void* stream);
+
+/* row = x_in + bias + v0 * y0 + v1 * y1  (y: T rows ld apart, may be null; v, bias: fp32 [W], null = ones / zeros) -> x_out (fp32,
+ * null only without parts; never x_in);  h = row / sqrt(mean(row^2) + eps) * (w + w_off) (w: fp32 [W]) -> h_out (T).  shift (fp32 [W]) !=
+ * null:  g = h + (h_prev - h) * shift -> g_out (T) with h_prev the unrounded h of the token before -- of the same launch inside a
+ * portion, state[req_rows[b]] (fp32 [rows, W]) for a portion's first token, zero at position 0; the last token of request b
+ * leaves its h in staging[b] (fp32 [batch, W]) for msgl_mix_commit_rows. */
+int msgl_mix_shift_norm(const float* x_in, float* x_out, const void* y0, int64_t ld0, const float* v0, const void* y1, int64_t ld1,
+                        const float* v1, const float* bias, const float* w, float w_off, const float* shift, void* h_out, void* g_out,
+                        const float* state, float* staging, const int* positions, const int* cu_q, const int* req_rows, int batch,
+                        float eps, int rows, int W, int dtype, void* stream);
+
+/* dst[l * dst_stride + slots[b] * W ..] = src[l * src_stride + b * W ..] for l < layers, b < batch (requests without new tokens
+ * are skipped); prev_tok != null: prev_tok[slots[b]] = ids[cu_q[b + 1] - 1]. */
+int msgl_mix_commit_rows(float* dst, int64_t dst_stride, const float* src, int64_t src_stride, int layers, const int* slots, int batch, int W,
+                         int* prev_tok, const int* ids, const int* cu_q, void* stream);
+
+/* Projection row [q: H x d | k: G x d | v: G x dv | ...] (+ bias: fp32, same layout, may be null): the first rot_dims entries of
+ * every q and k head turn (cos_sin and pairing as in msgl_mix_latent_prep), with unit != 0 every q and k head is divided by its
+ * root mean square; q -> q_out (fp32 [tokens, H * d]), k and v -> cache rows at out_loc ([slots, G * d], [slots, G * dv], T). */
+int msgl_mix_qk_prep(const void* proj, int64_t ld_proj, const float* bias, float* q_out, void* k_cache, void* v_cache, const int* out_loc,
+                     const int* positions, const float* cos_sin, int rot_dims, int interleaved, int unit, float eps, int tokens, int H,
+                     int G, int d, int dv, int dtype, void* stream);
+
+/* Causal attention without normalisation over keys: out[t, h] = out_scale * sum_{j <= t} sigmoid(c(scale q_h . k_j) + pb[h]) v_j,
+ * c(s) = softcap * tanh(s / softcap) (softcap <= 0: c(s) = s), query head h reads key/value head h / (H / G).  q: fp32 [tokens,
+ * H * d]; out: T, rows ld_out apart; requests as in msgl_mix_latent_attn.  `splits` > 1 cuts every request's keys into ranges whose
+ * partial sums (workspace: fp32, msgl_mix_sigmoid_attn_workspace_floats) a second launch adds. */
+int msgl_mix_sigmoid_attn_workspace_floats(int total_q, int H, int dv, int splits);
+int msgl_mix_sigmoid_attn(void* out, int64_t ld_out, const float* q, const void* k_cache, const void* v_cache, const int* table,
+                          int64_t table_stride, const int* req_rows, const int* seq_lens, const int* cu_q, int batch, int total_q, int H,
+                          int G, int d, int dv, float scale, float softcap, const float* pb, float out_scale, int dtype, int splits,
+                          float* workspace, void* stream);
+
+/* State-space recurrence per (request, head): dt = softplus(dt_raw[t, h] + dt_bias[h]); S <- exp(rate[h] dt) S + dt B x^T;
+ * y = S^T C + D[h] x.  xbc: fp32 rows [x: H x P | B: G x N | C: G x N] (head h reads group h / (H / G)); dt_raw: T rows ld_dt
+ * apart; state: fp32 [slots, H, N, P], row slots[b], zero for a request whose first new token is at position 0; rate = -exp(A_log).
+ * out: fp32 [tokens, H * P].  n_items > 0: chunks as in msgl_mix_lightning (a chunk is S_end = exp(rate * sum dt) S_start + L);
+ * scratch: fp32, n_items * H * (N * P + 1) floats. */
+int msgl_mix_ssd(float* out, const float* xbc, int64_t ld_x, const void* dt_raw, int64_t ld_dt, float* state, const float* rate,
+                 const float* dt_bias, const float* D, const int* cu_q, const int* seq_lens, const int* slots, int batch, int H, int G, int N,
+                 int P, int dtype, int n_items, const int* items, const int* item_first, float* scratch, void* stream);
+
+/* v = y * silu(z) (y fp32 [rows, N], z T rows ld_z apart); every one of `groups` equal parts of a row is divided by its own root
+ * mean square; out = v * w * out_scale (w fp32 [N]; out T, rows ld_out apart). */
+int msgl_mix_gate_group_norm(void* out, int64_t ld_out, const float* y, const void* z, int64_t ld_z, const float* w, float eps, int rows,
+                             int N, int groups, float out_scale, int dtype, void* stream);
+
+/* out = z > 0 ? a z^2 + z / 2 : b (exp(z) - 1 - z) + z / 2 with a = softplus(pq[0]), b = 1/2 + softplus(pq[1]) (pq: 2 floats on the
+ * device); z rows ldz apart, out rows of N. */
+int msgl_mix_xielu(void* out, const void* z, int64_t ldz, const float* pq, int rows, int N, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

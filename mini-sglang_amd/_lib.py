@@ -20,7 +20,7 @@ HIP_SO = LIB_DIR / "libmsgl_hip.so"
 COMM_SO = LIB_DIR / "libmsgl_comm.so"
 GEMM_SO = LIB_DIR / "libmsgl_gemm.so"
 MIX_SO = LIB_DIR / "libmsgl_mix.so"
-MIX_ABI_VERSION = 2
+MIX_ABI_VERSION = 3
 
 BF16, FP16, F32 = 0, 1, 2
 UNIQUE_ID_BYTES = 128
@@ -145,9 +145,9 @@ MIX_SIGNATURES = {
     "msgl_mix_abi_version": (_i, []),
     "msgl_mix_embed": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
     "msgl_mix_postnorm": (_i, [_p, _p, _p, _p, _i, _p, _p, _f, _f, _i, _i, _i, _p, _p, _i, _i, _i, _i, _p, _p, _p]),
-    "msgl_mix_latent_prep": (_i, [_p, _l, _p, _p, _p, _p, _p, _p, _f, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "msgl_mix_latent_prep": (_i, [_p, _l, _p, _p, _p, _p, _p, _p, _f, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "msgl_mix_latent_attn_workspace_floats": (_i, [_i, _i, _i, _i]),
-    "msgl_mix_latent_attn": (_i, [_p, _p, _p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p, _p]),
+    "msgl_mix_latent_attn": (_i, [_p, _p, _p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _f, _p, _i, _i, _p, _p]),
     "msgl_mix_lightning": (_i, [_p, _p, _l, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
     "msgl_mix_gated_norm": (_i, [_p, _p, _p, _l, _p, _f, _i, _i, _i, _p]),
     "msgl_mix_route": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
@@ -161,9 +161,18 @@ MIX_SIGNATURES = {
     "msgl_mix_kv_store": (_i, [_p, _p, _p, _p, _l, _i, _i, _i, _i, _p, _l, _p, _i, _i, _p]),
     "msgl_mix_window_attn_workspace_floats": (_i, [_i, _i, _i, _i]),
     "msgl_mix_window_attn": (_i, [_p, _p, _l, _i, _p, _p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p, _i, _i, _p, _p]),
-    "msgl_mix_short_conv": (_i, [_p, _p, _l, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "msgl_mix_short_conv": (_i, [_p, _p, _l, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "msgl_mix_delta_rule": (_i, [_p, _p, _p, _p, _l, _p, _l, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
     "msgl_mix_head_gated_norm": (_i, [_p, _p, _p, _l, _p, _f, _i, _i, _i, _i, _i, _p]),
+    "msgl_mix_embed_scaled": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _p, _f, _i, _i, _i, _i, _i, _i, _p]),
+    "msgl_mix_shift_norm": (_i, [_p, _p, _p, _l, _p, _p, _l, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _p, _p, _i, _f, _i, _i, _i, _p]),
+    "msgl_mix_commit_rows": (_i, [_p, _l, _p, _l, _i, _p, _i, _i, _p, _p, _p, _p]),
+    "msgl_mix_qk_prep": (_i, [_p, _l, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _p]),
+    "msgl_mix_sigmoid_attn_workspace_floats": (_i, [_i, _i, _i, _i]),
+    "msgl_mix_sigmoid_attn": (_i, [_p, _l, _p, _p, _p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _f, _p, _f, _i, _i, _p, _p]),
+    "msgl_mix_ssd": (_i, [_p, _p, _l, _p, _l, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
+    "msgl_mix_gate_group_norm": (_i, [_p, _l, _p, _p, _l, _p, _f, _i, _i, _i, _f, _i, _p]),
+    "msgl_mix_xielu": (_i, [_p, _p, _l, _p, _i, _i, _i, _p]),
 }
 
 

@@ -37,6 +37,7 @@ class HipAttnMetadata:
     plan: Optional[torch.Tensor] = None     # decode work list (device)
     chunks: Optional[tuple] = None          # recurrent layers: (items [n, 3], item_first [B + 1], n) of long portions cut in pieces
     delta_chunks: Optional[tuple] = None    # the same list at the delta-rule layers' piece size
+    ssd_chunks: Optional[tuple] = None      # the same list at the state-space layers' piece size
 
     def get_last_indices(self, bs: int) -> torch.Tensor:
         return self.cu_seqlens_q[1: 1 + bs] - 1
@@ -224,6 +225,7 @@ class MixAttnBackend:
 
     RECURRENT_CHUNK = 128
     DELTA_CHUNK = 256
+    SSD_CHUNK = 128
 
     def __init__(self, config: Any, ctx: Any = None, *, tp_size: int = 1) -> None:
         ctx = ctx if ctx is not None else _core.get_global_ctx()
@@ -234,6 +236,7 @@ class MixAttnBackend:
         self.capture_bs: List[int] = []
         self._cap: Optional[torch.Tensor] = None
         self._kinds = {getattr(s, "kind", "") for s in getattr(config, "layers", ())}
+        self._kinds |= {getattr(p, "kind", "") for s in getattr(config, "layers", ()) for p in (getattr(s, "left", None), getattr(s, "right", None)) if p}
 
     def prepare_metadata(self, batch: Any) -> None:
         reqs = batch.padded_reqs
@@ -248,6 +251,8 @@ class MixAttnBackend:
             lists.append(("chunks", self.RECURRENT_CHUNK))
         if int(q.max()) >= 2 * self.DELTA_CHUNK and self._kinds & {"delta", "channel_delta"}:
             lists.append(("delta_chunks", self.DELTA_CHUNK))
+        if int(q.max()) >= 2 * self.SSD_CHUNK and "state_space" in self._kinds:
+            lists.append(("ssd_chunks", self.SSD_CHUNK))
         pieces = [-(-q // c) for _, c in lists]
         extra = sum(3 * int(p.sum()) + bs + 1 for p in pieces)
         host = torch.empty(3 * bs + 1 + extra, dtype=torch.int32, pin_memory=True)

@@ -507,16 +507,16 @@ __global__ __launch_bounds__(256) void window_merge_kernel(T* __restrict__ out, 
 }
 
 // ------------------------------------------------------------------------------------------------ short convolution
-// One workgroup per token.  y[c] = silu(sum_j taps[c][j] in[pos - (n - 1) + j][c]); inputs of this portion come from `src`, earlier
+// One workgroup per token.  y[c] = silu(bias[c] + sum_j taps[c][j] in[pos - (n - 1) + j][c]) (bias may be null); inputs of this portion come from `src`, earlier
 // ones from the request's conv state (state[slot][s][c] = the input at position start - (n - 1) + s), positions < 0 are zero.
 // The first `unit_heads` groups of d channels are made unit vectors (x / sqrt(sum x^2 + 1e-6)); the first `scaled_heads` of them
 // are also multiplied by d^-1/2.
 template <typename T>
 __global__ __launch_bounds__(256) void short_conv_kernel(float* __restrict__ out, const T* __restrict__ src, int64_t ld_src,
-                                                         const T* __restrict__ taps, const T* __restrict__ state,
-                                                         const int* __restrict__ cu_q, const int* __restrict__ seq_lens,
-                                                         const int* __restrict__ slots, int batch, int C, int n, int unit_heads,
-                                                         int scaled_heads, int d) {
+                                                         const T* __restrict__ taps, const T* __restrict__ bias,
+                                                         const T* __restrict__ state, const int* __restrict__ cu_q,
+                                                         const int* __restrict__ seq_lens, const int* __restrict__ slots, int batch, int C,
+                                                         int n, int unit_heads, int scaled_heads, int d) {
   extern __shared__ float row[];  // C
   const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int b = request_of(cu_q, batch, t);
@@ -524,7 +524,7 @@ __global__ __launch_bounds__(256) void short_conv_kernel(float* __restrict__ out
   const int pos = seq_lens[b] - (cu_q[b + 1] - cu_q[b]) + local;
   const T* st_row = state + (size_t)slots[b] * (n - 1) * C;
   for (int c = tid; c < C; c += 256) {
-    float s = 0.f;
+    float s = bias ? ld(bias + c) : 0.f;
     for (int j = 0; j < n; ++j) {
       const int back = n - 1 - j;  // how many tokens before this one
       if (pos - back < 0) continue;
@@ -935,9 +935,9 @@ int msgl_mix_window_attn(void* out, const void* src, int64_t ld_src, int g_off, 
   return MSGL_MIX_OK;
 }
 
-int msgl_mix_short_conv(float* out, const void* src, int64_t ld_src, const void* taps, void* state, const int* cu_q, const int* seq_lens,
-                        const int* slots, int batch, int total, int C, int n, int unit_heads, int scaled_heads, int d, int dtype,
-                        void* stream) {
+int msgl_mix_short_conv(float* out, const void* src, int64_t ld_src, const void* taps, const void* bias, void* state, const int* cu_q,
+                        const int* seq_lens, const int* slots, int batch, int total, int C, int n, int unit_heads, int scaled_heads, int d,
+                        int dtype, void* stream) {
   MIX_REQUIRE(out && src && taps && cu_q && seq_lens && slots && dtype_ok(dtype), "short_conv: null pointer / dtype");
   MIX_REQUIRE(batch >= 0 && total >= 0 && C >= 1 && n >= 1 && n <= 17 && ld_src >= C && (n == 1 || state),
               "short_conv: bad sizes C %d taps %d", C, n);
@@ -947,8 +947,8 @@ int msgl_mix_short_conv(float* out, const void* src, int64_t ld_src, const void*
   const size_t lds = (size_t)C * sizeof(float);
   hipStream_t s = static_cast<hipStream_t>(stream);
   DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)short_conv_kernel<T>, lds) == 0, "short_conv: row of %d does not fit LDS", C);
-             hipLaunchKernelGGL(short_conv_kernel<T>, dim3(total), dim3(256), lds, s, out, cp<T>(src), ld_src, cp<T>(taps), cp<T>(state),
-                                cu_q, seq_lens, slots, batch, C, n, unit_heads, scaled_heads, d);
+             hipLaunchKernelGGL(short_conv_kernel<T>, dim3(total), dim3(256), lds, s, out, cp<T>(src), ld_src, cp<T>(taps), cp<T>(bias),
+                                cp<T>(state), cu_q, seq_lens, slots, batch, C, n, unit_heads, scaled_heads, d);
              if (n > 1) hipLaunchKernelGGL(conv_state_kernel<T>, dim3((C + 255) / 256, batch), dim3(256), 0, s, mp<T>(state), cp<T>(src),
                                            ld_src, cu_q, slots, C, n);)
   MIX_LAUNCHED("short_conv");

@@ -52,12 +52,13 @@ __global__ __launch_bounds__(256) void postnorm_kernel(const float* __restrict__
 // ------------------------------------------------------------------------------------------------ latent prep
 // One workgroup per token.  proj row = [ q: H x (d + r) | (has_kv) latent R | shared rotated key part r ].
 // cos_sin row p = [cos(p f_i) * amp, i < rd/2 | sin(p f_i) * amp]; the first rd entries of a rotated part turn, the rest pass.
+// Entry i is paired with i + rd / 2, or, with `interleaved`, entries 2i and 2i + 1 form pair i.
 template <typename T>
 __global__ __launch_bounds__(256) void latent_prep_kernel(const T* __restrict__ proj, int64_t ld_proj, float* __restrict__ q_abs,
                                                           T* __restrict__ cache, const int* __restrict__ out_loc,
                                                           const int* __restrict__ positions, const float* __restrict__ cos_sin,
                                                           const T* __restrict__ c_norm_w, float eps, int H, int d, int r, int rd, int R,
-                                                          int has_kv) {
+                                                          int has_kv, int interleaved) {
   __shared__ float red[4];
   const int t = blockIdx.x;
   const T* row = proj + (size_t)t * ld_proj;
@@ -69,7 +70,10 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const T* __restrict__ 
     const int hh = i / r, j = i - hh * r;
     const T* qr = row + (size_t)hh * (d + r) + d;
     float v = ld(qr + j);
-    if (j < rd) {
+    if (j < rd && interleaved) {
+      const float c = cs[j >> 1], s = cs[half + (j >> 1)], other = ld(qr + (j ^ 1));
+      v = (j & 1) ? v * c + other * s : v * c - other * s;
+    } else if (j < rd) {
       const int pidx = j < half ? j : j - half;
       const float c = cs[pidx], s = cs[half + pidx];
       const float u0 = ld(qr + pidx), v0 = ld(qr + pidx + half);
@@ -89,7 +93,10 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const T* __restrict__ 
   for (int i = threadIdx.x; i < R; i += 256) st(dst + i, ld(kv + i) * inv * ld(c_norm_w + i));
   for (int j = threadIdx.x; j < r; j += 256) {
     float v = ld(kv + R + j);
-    if (j < rd) {
+    if (j < rd && interleaved) {
+      const float c = cs[j >> 1], s = cs[half + (j >> 1)], other = ld(kv + R + (j ^ 1));
+      v = (j & 1) ? v * c + other * s : v * c - other * s;
+    } else if (j < rd) {
       const int pidx = j < half ? j : j - half;
       const float c = cs[pidx], s = cs[half + pidx];
       const float u0 = ld(kv + R + pidx), v0 = ld(kv + R + pidx + half);
@@ -131,6 +138,15 @@ __device__ __forceinline__ void find_group(const int* __restrict__ cu_q, int B, 
   __syncthreads();
 }
 
+// A sink is one more term exp(sink[h]) in a head's softmax denominator, with no key and no value.  With running maximum m
+// over the keys and M = max(m, sink): out = f o / (f l + w), f = exp(m - M), w = exp(sink - M)  (no sink: f = 1, w = 0).
+__device__ __forceinline__ float sink_factor(const float* __restrict__ sink, int head, float m) {
+  return (sink && sink[head] > m) ? expf(m - sink[head]) : 1.f;
+}
+__device__ __forceinline__ float sink_weight(const float* __restrict__ sink, int head, float m) {
+  return sink ? (sink[head] > m ? 1.f : expf(sink[head] - m)) : 0.f;
+}
+
 // Query rows are (token, head) pairs; all heads read the same key row (latent R | rotated r) and the same value row
 // (the latent).  A workgroup = 16 query rows (QT tokens of one request x HB heads) x 16 lanes; keys in tiles of KT through
 // LDS as fp32; online softmax per row in fp32; output = softmax-weighted latent, fp32.
@@ -142,7 +158,8 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(float* __restrict__ ou
                                                           const T* __restrict__ cache, const int* __restrict__ table,
                                                           int64_t table_stride, const int* __restrict__ req_rows,
                                                           const int* __restrict__ seq_lens, const int* __restrict__ cu_q, int B,
-                                                          int H, int dk, int dv, float scale, int QT, int HB, int KT) {
+                                                          int H, int dk, int dv, float scale, int QT, int HB, int KT,
+                                                          const float* __restrict__ sink) {
   extern __shared__ float lds[];
   const int qs = dk + 1;
   float* sq = lds;                       // [16][dk + 1]
@@ -220,7 +237,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(float* __restrict__ ou
     }
   }
   if (!valid) return;
-  const float inv = 1.0f / lsum;
+  const float inv = sink_factor(sink, head, m) / (sink_factor(sink, head, m) * lsum + sink_weight(sink, head, m));
 #pragma unroll
   for (int i = 0; i < kAttnMaxC; ++i) {
     const int c = l + 16 * i;
@@ -900,7 +917,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(float* __restrict
                                                                const int* __restrict__ table, int64_t table_stride,
                                                                const int* __restrict__ req_rows, const int* __restrict__ seq_lens,
                                                                const int* __restrict__ cu_q, int B, int H, int dk, int dv, float scale,
-                                                               int QT, int HB, int splits, int vec) {
+                                                               int QT, int HB, int splits, int vec, const float* __restrict__ sink) {
   constexpr int KS = KC * 32 + 8;
   extern __shared__ __attribute__((aligned(16))) uint16_t sk[];  // [kAKT][KS]
   __shared__ int s_req, s_tok0, s_cnt[256];
@@ -1067,7 +1084,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(float* __restrict
   if (!valid) return;
   const size_t row = (size_t)tok * H + head;
   if (splits == 1) {
-    const float inv = 1.0f / lsum;
+    const float inv = sink_factor(sink, head, m) / (sink_factor(sink, head, m) * lsum + sink_weight(sink, head, m));
 #pragma unroll
     for (int vt = 0; vt < VC; ++vt)
 #pragma unroll
@@ -1091,9 +1108,11 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(float* __restrict
   }
 }
 
-// out[row] = sum_z e^(m_z - m*) o_z / sum_z e^(m_z - m*) l_z, splits in order; a split without keys has l = 0 and m = -inf
+// out[row] = sum_z e^(m_z - m*) o_z / (sum_z e^(m_z - m*) l_z + e^(sink - m*)), splits in order; a split without keys has l = 0
+// and m = -inf; without a sink its term is absent
 __global__ __launch_bounds__(64) void latent_attn_merge_kernel(float* __restrict__ out, const float* __restrict__ part_o,
-                                                               const float* __restrict__ part_ml, int splits, int dv) {
+                                                               const float* __restrict__ part_ml, int splits, int dv,
+                                                               const float* __restrict__ sink, int H) {
   __shared__ float sw[1024];  // per split: its max, then its weight e^(m_z - m*)
   __shared__ float sl[1024];
   const size_t row = blockIdx.x;
@@ -1102,9 +1121,9 @@ __global__ __launch_bounds__(64) void latent_attn_merge_kernel(float* __restrict
     sl[z] = part_ml[(row * splits + z) * 2 + 1];
   }
   __syncthreads();
-  float ms = -INFINITY;
+  float ms = sink ? sink[row % H] : -INFINITY;  // the sink joins the maximum and the denominator like one more range
   for (int z = 0; z < splits; ++z) ms = fmaxf(ms, sw[z]);
-  float l = 0.f;
+  float l = sink ? __expf(sink[row % H] - ms) : 0.f;
   for (int z = 0; z < splits; ++z) l += sw[z] > -INFINITY ? sl[z] * __expf(sw[z] - ms) : 0.f;
   __syncthreads();
   for (int z = threadIdx.x; z < splits; z += 64) sw[z] = sw[z] > -INFINITY ? __expf(sw[z] - ms) : 0.f;
@@ -1166,7 +1185,7 @@ int msgl_mix_postnorm(const float* x_in, float* x_out, void* h_out, const void* 
 
 int msgl_mix_latent_prep(const void* proj, int64_t ld_proj, float* q_abs, void* cache, const int* out_loc, const int* positions,
                          const float* cos_sin, const void* c_norm_w, float eps, int tokens, int H, int d, int r, int rot_dims, int R,
-                         int has_kv, int dtype, void* stream) {
+                         int has_kv, int interleaved, int dtype, void* stream) {
   MIX_REQUIRE(proj && q_abs && positions && cos_sin && dtype_ok(dtype), "latent_prep: null pointer / dtype");
   MIX_REQUIRE(H >= 1 && d >= 0 && r >= 0 && R >= 1 && rot_dims >= 0 && rot_dims <= r && rot_dims % 2 == 0,
               "latent_prep: bad sizes H %d d %d r %d rot %d R %d", H, d, r, rot_dims, R);
@@ -1175,7 +1194,7 @@ int msgl_mix_latent_prep(const void* proj, int64_t ld_proj, float* q_abs, void* 
   if (tokens == 0) return MSGL_MIX_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   DISPATCH_T(dtype, hipLaunchKernelGGL(latent_prep_kernel<T>, dim3(tokens), dim3(256), 0, s, cp<T>(proj), ld_proj, q_abs, mp<T>(cache),
-                                       out_loc, positions, cos_sin, cp<T>(c_norm_w), eps, H, d, r, rot_dims, R, has_kv);)
+                                       out_loc, positions, cos_sin, cp<T>(c_norm_w), eps, H, d, r, rot_dims, R, has_kv, interleaved);)
   MIX_LAUNCHED("latent_prep");
   return MSGL_MIX_OK;
 }
@@ -1185,8 +1204,8 @@ int msgl_mix_latent_attn_workspace_floats(int total_q, int H, int dv, int splits
 }
 
 int msgl_mix_latent_attn(float* out, const float* q_abs, const void* cache, const int* table, int64_t table_stride, const int* req_rows,
-                         const int* seq_lens, const int* cu_q, int batch, int total_q, int H, int dk, int dv, float scale, int dtype,
-                         int splits, float* workspace, void* stream) {
+                         const int* seq_lens, const int* cu_q, int batch, int total_q, int H, int dk, int dv, float scale,
+                         const float* sink, int dtype, int splits, float* workspace, void* stream) {
   MIX_REQUIRE(out && q_abs && cache && table && req_rows && seq_lens && cu_q && dtype_ok(dtype), "latent_attn: null pointer / dtype");
   MIX_REQUIRE(batch >= 1 && total_q >= 0 && H >= 1 && dv >= 1 && dk >= dv, "latent_attn: bad sizes");
   MIX_REQUIRE(splits >= 1 && splits <= 1024 && (splits == 1 || workspace), "latent_attn: %d splits need a workspace", splits);
@@ -1207,10 +1226,10 @@ int msgl_mix_latent_attn(float* out, const float* q_abs, const void* cache, cons
     const size_t lds = (size_t)kAKT * (KC * 32 + 8) * sizeof(uint16_t);                                                                \
     MIX_REQUIRE(ensure_lds((const void*)latent_attn_mfma_kernel<KC, VC>, lds) == 0, "latent_attn: LDS request refused");               \
     hipLaunchKernelGGL((latent_attn_mfma_kernel<KC, VC>), grid, dim3(256), lds, s, out, part_o, part_ml, q_abs, cp<bf16_t>(cache), table, \
-                       table_stride, req_rows, seq_lens, cu_q, batch, H, dk, dv, scale, QT, HB, splits, vec);                          \
+                       table_stride, req_rows, seq_lens, cu_q, batch, H, dk, dv, scale, QT, HB, splits, vec, sink);                    \
     MIX_LAUNCHED("latent_attn (matrix cores)");                                                                                        \
     if (splits > 1) {                                                                                                                  \
-      hipLaunchKernelGGL(latent_attn_merge_kernel, dim3(total_q * H), dim3(64), 0, s, out, part_o, part_ml, splits, dv);               \
+      hipLaunchKernelGGL(latent_attn_merge_kernel, dim3(total_q * H), dim3(64), 0, s, out, part_o, part_ml, splits, dv, sink, H);       \
       MIX_LAUNCHED("latent_attn merge");                                                                                               \
     }                                                                                                                                  \
     return MSGL_MIX_OK;                                                                                                                \
@@ -1234,7 +1253,7 @@ int msgl_mix_latent_attn(float* out, const float* q_abs, const void* cache, cons
   const int groups = (total_q + QT - 1) / QT + batch;  // every request may end with one partial group
   DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)latent_attn_kernel<T>, lds) == 0, "latent_attn: LDS request refused");
              hipLaunchKernelGGL(latent_attn_kernel<T>, dim3(groups, (H + HB - 1) / HB), dim3(256), lds, s, out, q_abs, cp<T>(cache), table,
-                                table_stride, req_rows, seq_lens, cu_q, batch, H, dk, dv, scale, QT, HB, KT);)
+                                table_stride, req_rows, seq_lens, cu_q, batch, H, dk, dv, scale, QT, HB, KT, sink);)
   MIX_LAUNCHED("latent_attn");
   return MSGL_MIX_OK;
 }

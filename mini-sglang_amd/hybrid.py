@@ -34,7 +34,26 @@ delta / channel_delta   q, k, v pass a short causal convolution over time (+ SiL
 feed-forward       dense with a polynomial activation of row-normalised powers, or routed experts silu(W_g h) * (W_u h)
                    chosen by the largest router logits (softmax over the chosen logits only).
 
-Kernels: csrc/seqmix.hip and csrc/mix_delta.hip through mixops.py; plain projections through the library GEMM (mixops.linear).
+A third scheme, `parallel_shift` (the Givavik design), has ONE norm per layer that feeds the mixer and the feed-forward side by side:
+
+stream             x_0 = s_e embed[token] + pair[(previous token * m_p + token * m_c) mod B] (row B for a sequence's first token);
+                   per layer  h = rms_unit(x) (1 + w),  g = h + (h of the token before - h) * shift  (zero before the first token),
+                   x <- x + ls1 * mixer(g) + ls2 * ff(h);  final norm, then the LM head matrix.  Per request the state rows keep
+                   the last token id and, for every layer, the last h (fp32).
+latent attention   as above, with the rotated parts paired (2i, 2i + 1) and a learned sink per head: one more term exp(sink_h) in
+                   the softmax denominator that has no key and no value.
+parallel           two mixers on the same g, their results scaled and added:
+  sigmoid attention  H query heads over G key/value heads with projection biases, rotation of the leading entries of each head,
+                   q and k divided by their root mean square, score = cap tanh(scale q.k / cap), weight of a visible key =
+                   sigmoid(score + b_h), no normalisation over keys.  Cached per token: k [G d] and v [G dv].
+  state space      Mamba-2: in-projection [z | x | B | C | dt], causal convolution + SiLU over x, B, C, dt = softplus(dt + bias),
+                   S <- exp(-exp(A) dt) S + dt B x^T, y = S^T C + D x, y * silu(z) RMS-normed in equal groups, output projection.
+                   State per request: S in fp32 and the last taps - 1 inputs of the convolution.
+                   Both mixers share one input projection and one output projection (their outputs side by side in one row).
+feed-forward       W_down xielu(W_up h) with two learned numbers per layer.
+
+Kernels: csrc/seqmix.hip, csrc/mix_delta.hip and csrc/mix_par.hip through mixops.py; plain projections through the library GEMM
+(mixops.linear).
 """
 from __future__ import annotations
 
@@ -63,12 +82,14 @@ class MoeSpec:
 @dataclass(frozen=True)
 class DenseFfSpec:
     ff: int
-    act: str = "poly_norm"          # c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3 with N = divide a row by its root mean square
+    act: str = "poly_norm"          # "poly_norm": c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3 with N = divide a row by its root mean square;
+                                    # "xielu": softplus(p) z^2 + z / 2 above zero, (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2 below
 
 
 @dataclass(frozen=True)
 class LayerSpec:
-    kind: str                       # "latent_attention" | "lightning" | "attention" | "delta" | "channel_delta"
+    kind: str                       # "latent_attention" | "lightning" | "attention" | "delta" | "channel_delta" | "parallel";
+                                    # inside a "parallel" pair: "sigmoid_attention" | "state_space"
     heads: int
     dim: int                        # unrotated query/key size per head (lightning: query/key size)
     vdim: int
@@ -87,10 +108,20 @@ class LayerSpec:
     conv: int = 1                   # delta kinds: taps of the causal convolution over q, k, v
     decay_rank: int = 0             # channel_delta: inner sizes of the two-step decay and gate projections
     gate_rank: int = 0
+    interleaved: bool = False       # rotation pairs entries (2i, 2i + 1) instead of (i, i + half)
+    sink: bool = False              # latent attention: a learned term per head in the softmax denominator
+    softcap: float = 0.0            # sigmoid attention: score <- cap tanh(score / cap); 0 = none
+    norm_groups: int = 1            # state space: the gated output is RMS-normed in this many equal parts
+    left: Optional["LayerSpec"] = None   # parallel: the two mixers that read the same input, and the scales of their sum
+    right: Optional["LayerSpec"] = None
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    # state space: heads x vdim = inner size, dim = state size per head, kv_heads = groups of B / C, conv = taps
 
     @property
     def recurrent(self) -> bool:
-        return self.kind in ("lightning", "delta", "channel_delta")
+        return self.kind in ("lightning", "delta", "channel_delta", "state_space") or \
+            (self.kind == "parallel" and (self.left.recurrent or self.right.recurrent))
 
 
 @dataclass(frozen=True)
@@ -104,7 +135,11 @@ class HybridConfig:
     max_position: int = 1 << 20
     name: str = "Nidorax"
     residual: str = "post_norm"     # "post_norm": x <- norm(alpha x + f(x)), weights stored as offsets from one, tied head;
-                                    # "pre_norm_depth": x + f(norm(x)), depth-averaged history, normed embedding, own head
+                                    # "pre_norm_depth": x + f(norm(x)), depth-averaged history, normed embedding, own head;
+                                    # "parallel_shift": x + ls1 mixer(shift(norm(x))) + ls2 ff(norm(x)), own head
+    embed_scale: float = 1.0        # parallel_shift: the embedding row is multiplied by this
+    pair_embed: Optional[Tuple[int, int, int]] = None  # (buckets, multiplier of the previous id, multiplier of the id) of the pair table
+    token_shift: bool = False       # every layer's mixer reads a blend of this token's and the previous token's normed row
 
     @property
     def num_layers(self) -> int:
@@ -193,6 +228,62 @@ def bedarax_config(cfg: Dict[str, Any], shapes: Optional[Dict[str, Tuple[int, ..
                         rms_norm_eps=float(cfg["norm"]["eps"]), name=name, residual="pre_norm_depth")
 
 
+def _rot(m: Dict[str, Any], default_dims: int) -> Tuple[int, float]:
+    rot = m.get("rot") or {}
+    return int(rot.get("dims", default_dims)), float(rot.get("base", 10000.0))
+
+
+def givavik_config(cfg: Dict[str, Any], name: str = "Givavik") -> HybridConfig:
+    """config.json of a Givavik model -> HybridConfig."""
+    layers: List[LayerSpec] = []
+    for i, entry in enumerate(cfg["layers"]):
+        m, kind, mlp = entry["mixer"], entry["type"], entry.get("mlp")
+        ff = None
+        if mlp is not None:
+            if mlp.get("kind") != "dense":
+                raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+            ff = DenseFfSpec(ff=int(mlp["ff"]), act="xielu")
+        if kind == "latent_attention":
+            dims, base = _rot(m, int(m["rot_dim"]))
+            layers.append(LayerSpec(
+                kind="latent_attention", heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), rot_dim=int(m["rot_dim"]),
+                kv_rank=int(m["kv_rank"]), kv_from=None if m.get("kv_from") is None else int(m["kv_from"]), scale=float(m["scale"]),
+                rot_dims=dims, rot_base=base, interleaved=True, sink=True, mlp=ff))
+        elif kind == "parallel":
+            a, b = m["left"], m["right"]
+            H, G = int(a["heads"]), int(a.get("kv_heads", a["heads"]))
+            dims, base = _rot(a, 0)
+            left = LayerSpec(kind="sigmoid_attention", heads=H, kv_heads=G, dim=int(a["dim"]), vdim=int(a["vdim"]), scale=float(a["scale"]),
+                             softcap=float(a.get("softcap") or 0.0), rot_dims=dims, rot_base=base, interleaved=True)
+            Hs, Gs = int(b["heads"]), int(b.get("groups", 1))
+            right = LayerSpec(kind="state_space", heads=Hs, kv_heads=Gs, dim=int(b["state"]), vdim=int(b["vdim"]), conv=int(b["conv"]),
+                              norm_groups=int(b.get("norm_groups", 1)))
+            if H % G or Hs % Gs or (Hs * right.vdim) % right.norm_groups or dims % 2 or dims > left.dim:
+                raise ValueError(f"layer {i}: head / group / rotation sizes do not divide")
+            layers.append(LayerSpec(kind="parallel", heads=H, dim=left.dim, vdim=left.vdim, left=left, right=right,
+                                    left_scale=float(m.get("left_scale", 1.0)), right_scale=float(m.get("right_scale", 1.0)), mlp=ff))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+    for i, s in enumerate(layers):
+        if s.kind == "latent_attention" and s.kv_from is not None:
+            o = layers[s.kv_from] if 0 <= s.kv_from < i else None
+            if o is None or o.kind != "latent_attention" or o.kv_from is not None or \
+                    (o.kv_rank, o.rot_dim, o.rot_dims, o.rot_base) != (s.kv_rank, s.rot_dim, s.rot_dims, s.rot_base):
+                raise ValueError(f"layer {i}: kv_from = {s.kv_from} is not an earlier latent layer with its own keys of equal size and rotation")
+    e = cfg.get("embedding") or {}
+    bg = e.get("bigram")
+    pair = None if not bg else (int(bg["buckets"]), int(bg["mul_prev"]), int(bg["mul_cur"]))
+    return HybridConfig(vocab_size=int(cfg["vocab"]), hidden_size=int(cfg["width"]), layers=tuple(layers), rms_norm_eps=float(cfg["norm"]["eps"]),
+                        name=name, residual="parallel_shift", embed_scale=float(e.get("scale", 1.0)), pair_embed=pair, token_shift=True)
+
+
+def plain_rotary_table(dims: int, base: float, max_position: int, device) -> torch.Tensor:
+    """fp32 [max_position, dims] = cos | sin of position * base^(-2i / dims), i < dims / 2; angles in float64, rounded once."""
+    f = float(base) ** (-2.0 * torch.arange(dims // 2, dtype=torch.float64) / dims)
+    ang = torch.arange(max_position, dtype=torch.float64)[:, None] * f[None, :]
+    return torch.cat((ang.cos(), ang.sin()), dim=-1).to(torch.float32).to(device)
+
+
 def rotary_table(spec: LayerSpec, max_position: int, device) -> torch.Tensor:
     """fp32 [max_position, rot_dims] = cos | sin of the layer's (scaled) rotary angles, amplitude folded in."""
     sc = dict(spec.rot_scaling) if spec.rot_scaling else None
@@ -205,7 +296,8 @@ def rotary_table(spec: LayerSpec, max_position: int, device) -> torch.Tensor:
 
 class _Layer:
     __slots__ = ("spec", "w_in", "o", "norm1", "norm2", "uk_t", "uv", "c_norm", "cos_sin", "out_norm", "decay", "router",
-                 "bias", "up", "down", "talk", "lam", "taps", "rate", "dt_bias", "a2", "g2", "act", "depth_w")
+                 "bias", "up", "down", "talk", "lam", "taps", "rate", "dt_bias", "a2", "g2", "act", "depth_w",
+                 "sink", "ls1", "ls2", "shift", "in_bias", "out_bias", "pb", "skip", "conv_b", "sum_bias")
 
     def __init__(self, spec: LayerSpec) -> None:
         self.spec = spec
@@ -233,26 +325,60 @@ class HybridDecoder:
 
         W = cfg.hidden_size
         self.pre_norm = cfg.residual == "pre_norm_depth"
-        self.embed_norm = self.head = None
+        self.parallel = cfg.residual == "parallel_shift"
+        self.embed_norm = self.head = self.pair_table = None
         self.embed = w(cfg.vocab_size, W, std=1.0)
         self.final_norm = w(W, std=0.1)
         self.layers: List[_Layer] = []
         tables: Dict[tuple, torch.Tensor] = {}
+
+        def f32(*shape, std=init_std, mean=0.0):  # what the kernels read as fp32: norm offsets, per-column scales, biases, rates
+            return mean + torch.randn(shape, generator=g, device=device, dtype=torch.float32) * std
+
+        def plain_table(dims, base):
+            key = ("plain", dims, base)
+            if key not in tables:
+                tables[key] = plain_rotary_table(dims, base, self.max_position, device)
+            return tables[key]
+
         for spec in cfg.layers:
             L = _Layer(spec)
             H, d, dv = spec.heads, spec.dim, spec.vdim
             L.norm1 = w(W, std=0.1)
-            if spec.kind == "latent_attention":
+            if self.parallel:
+                L.norm1, L.ls1, L.ls2 = f32(W, std=0.1), f32(W, std=0.2, mean=1.0), f32(W, std=0.2, mean=1.0)
+                L.shift = f32(W, std=0.2, mean=0.5) if cfg.token_shift else None
+            if spec.kind == "parallel":
+                a, b = spec.left, spec.right
+                G, Gs, N = a.kv_heads, b.kv_heads, b.dim
+                n_left, inner = (H + G) * d + G * dv, b.heads * b.vdim
+                # one input projection: q | k | v of the attention, then z | x | B | C | dt of the state-space layer
+                L.w_in = w(n_left + 2 * inner + 2 * Gs * N + b.heads, W, std=W ** -0.5)
+                L.in_bias = f32(n_left, std=0.1)
+                L.pb = f32(H, std=1.0, mean=-2.0)
+                L.cos_sin = plain_table(a.rot_dims, a.rot_base) if a.rot_dims else None
+                L.taps = w(inner + 2 * Gs * N, b.conv, std=b.conv ** -0.5)
+                L.conv_b = w(inner + 2 * Gs * N, std=0.1)
+                L.dt_bias, L.rate, L.skip = f32(b.heads, std=0.5), -torch.exp(f32(b.heads, std=0.5)), f32(b.heads, std=0.5, mean=1.0)
+                L.out_norm = f32(inner, std=0.1, mean=1.0)
+                # one output projection over the row [attention heads | state-space channels]
+                L.o = w(W, H * dv + inner, std=(H * dv + inner) ** -0.5)
+                L.out_bias = f32(W, std=0.1)
+            elif spec.kind == "latent_attention":
                 r, R = spec.rot_dim, spec.kv_rank
                 L.w_in = w(H * (d + r) + (0 if spec.kv_from is not None else R + r), W, std=W ** -0.5)
                 L.uk_t = w(H, R, d, std=R ** -0.5)   # W_uk per head, transposed: q_abs = q_unrotated @ uk_t[h]^T
                 L.uv = w(H, dv, R, std=R ** -0.5)
                 L.o = w(W, H * dv, std=(H * dv) ** -0.5)
                 L.c_norm = None if spec.kv_from is not None else (1.0 + w(R, std=0.1).float()).to(dtype)
-                key = (spec.rot_dims, spec.rot_base, spec.rot_scaling)
-                if key not in tables:
-                    tables[key] = rotary_table(spec, self.max_position, device)
-                L.cos_sin = tables[key]
+                L.sink = f32(H, std=1.0) if spec.sink else None
+                if spec.interleaved:
+                    L.cos_sin = plain_table(spec.rot_dims, spec.rot_base)
+                else:
+                    key = (spec.rot_dims, spec.rot_base, spec.rot_scaling)
+                    if key not in tables:
+                        tables[key] = rotary_table(spec, self.max_position, device)
+                    L.cos_sin = tables[key]
             elif spec.kind == "lightning":
                 L.w_in = w(2 * H * d + 2 * H * dv, W, std=W ** -0.5)  # q | k | v | gate
                 L.o = w(W, H * dv, std=(H * dv) ** -0.5)
@@ -285,10 +411,10 @@ class HybridDecoder:
                 L.up = w(m.experts, (2 if m.gated else 1) * m.ff, W, std=W ** -0.5)  # gated: every expert's gate rows, then its up rows
                 L.down = w(m.experts, W, m.ff, std=m.ff ** -0.5)
             elif isinstance(m, DenseFfSpec):
-                L.norm2 = w(W, std=0.1)
+                L.norm2 = None if self.parallel else w(W, std=0.1)
                 L.up = w(m.ff, W, std=W ** -0.5)
                 L.down = w(W, m.ff, std=m.ff ** -0.5)
-                L.act = torch.tensor([1.0, 0.3, 0.1, 0.01], dtype=torch.float32, device=device)
+                L.act = torch.tensor([0.3, -0.4] if m.act == "xielu" else [1.0, 0.3, 0.1, 0.01], dtype=torch.float32, device=device)
             if self.pre_norm:
                 L.norm1, L.norm2 = (1.0 + L.norm1.float()).to(dtype), None if L.norm2 is None else (1.0 + L.norm2.float()).to(dtype)
                 c = torch.full((len(self.layers) + 2,), 0.1, dtype=torch.float32, device=device)
@@ -299,17 +425,31 @@ class HybridDecoder:
             self.final_norm = (1.0 + self.final_norm.float()).to(dtype)
             self.embed_norm = (1.0 + w(W, std=0.1).float()).to(dtype)
             self.head = w(cfg.vocab_size, W, std=W ** -0.5)
+        if self.parallel:
+            self.final_norm = f32(W, std=0.1)
+            self.head = w(cfg.vocab_size, W, std=W ** -0.5)
+            if cfg.pair_embed is not None:
+                self.pair_table = w(cfg.pair_embed[0] + 1, W, std=1.0)
+            self._derive()
 
     # ------------------------------------------------------------------ weights
+    def _derive(self) -> None:
+        """What the kernels read that is a function of loaded tensors: a pair layer's output bias as it enters the residual sum
+        (the attention's projection bias times the attention's scale times the layer scale of the mixer)."""
+        for L in self.layers:
+            if L.spec.kind == "parallel":
+                L.sum_bias = (L.out_bias * L.spec.left_scale * L.ls1).contiguous()
+
     def _tensors(self):
         yield self.embed
         yield self.final_norm
-        for t in (self.embed_norm, self.head):
+        for t in (self.embed_norm, self.head, self.pair_table):
             if t is not None:
                 yield t
         for L in self.layers:
             for k in ("w_in", "o", "norm1", "norm2", "uk_t", "uv", "c_norm", "out_norm", "router", "bias", "up", "down", "talk", "lam",
-                      "taps", "rate", "dt_bias", "a2", "g2", "act", "depth_w"):
+                      "taps", "rate", "dt_bias", "a2", "g2", "act", "depth_w", "sink", "ls1", "ls2", "shift", "in_bias", "out_bias", "pb",
+                      "skip", "conv_b"):
                 t = getattr(L, k)
                 if t is not None:
                     yield t
@@ -336,13 +476,38 @@ class HybridDecoder:
         if self.pre_norm:
             put(self.embed_norm, state["embed.norm"])
             put(self.head, state["head"])
+        if self.parallel:
+            put(self.head, state["head"])
+            if self.pair_table is not None:
+                put(self.pair_table, state["bigram"])
         for i, L in enumerate(self.layers):
             s, p = L.spec, f"l{i}.mix."
             H, d, dv = s.heads, s.dim, s.vdim
             put(L.norm1, state[f"l{i}.norm1"])
             if L.depth_w is not None:
                 put(L.depth_w, state[f"l{i}.dwa"])
-            if s.kind == "attention":
+            if self.parallel:
+                put(L.ls1, state[f"l{i}.ls1"])
+                if s.mlp is not None:
+                    put(L.ls2, state[f"l{i}.ls2"])
+                if L.shift is not None:
+                    put(L.shift, state[f"l{i}.shift"])
+            if L.sink is not None:
+                put(L.sink, state[p + "sink"])
+            if s.kind == "parallel":
+                a, b = p + "left.", p + "right."
+                put(L.w_in, torch.cat([state[a + "q"], state[a + "k"], state[a + "v"], state[b + "in"]], dim=0))
+                put(L.in_bias, torch.cat([state[a + "q.b"], state[a + "k.b"], state[a + "v.b"]], dim=0))
+                put(L.pb, state[a + "pb"])
+                put(L.taps, state[b + "conv"])
+                put(L.conv_b, state[b + "conv.b"])
+                put(L.dt_bias, state[b + "dt_bias"])
+                put(L.rate, -torch.exp(state[b + "A_log"].to(torch.float32)))
+                put(L.skip, state[b + "D"])
+                put(L.out_norm, state[b + "norm"])
+                put(L.o, torch.cat([state[a + "o"], state[b + "o"]], dim=1))
+                put(L.out_bias, state[a + "o.b"])
+            elif s.kind == "attention":
                 put(L.w_in, torch.cat([state[p + "q"], state[p + "k"], state[p + "v"], state[p + "g"]], dim=0))
                 put(L.talk, state[p + "talk"])
                 put(L.lam, state[p + "vmix"].reshape(1) if (p + "vmix") in state else torch.zeros(1))
@@ -366,13 +531,15 @@ class HybridDecoder:
             else:
                 put(L.w_in, torch.cat([state[p + "q"], state[p + "k"], state[p + "v"], state[p + "g"]], dim=0))
                 put(L.out_norm, state[p + "norm"])
-            put(L.o, state[p + "o"])
-            if s.mlp is None and f"l{i}.norm2" in state and not self.pre_norm:  # no feed-forward, but a second norm all the same
+            if s.kind != "parallel":
+                put(L.o, state[p + "o"])
+            if s.mlp is None and f"l{i}.norm2" in state and not self.pre_norm and not self.parallel:  # no feed-forward, but a second norm
                 L.norm2 = torch.empty_like(L.norm1)
                 put(L.norm2, state[f"l{i}.norm2"])
             if isinstance(s.mlp, DenseFfSpec):
                 q = f"l{i}.mlp."
-                put(L.norm2, state[f"l{i}.norm2"])
+                if L.norm2 is not None:
+                    put(L.norm2, state[f"l{i}.norm2"])
                 put(L.up, state[q + "up"])
                 put(L.down, state[q + "down"])
                 put(L.act, state[q + "act"])
@@ -393,19 +560,42 @@ class HybridDecoder:
                     L.bias = None
                 put(L.up, torch.stack([state[f"{q}e{e}.up"] for e in range(s.mlp.experts)]))
                 put(L.down, torch.stack([state[f"{q}e{e}.down"] for e in range(s.mlp.experts)]))
+        self._derive()
 
     def export_state(self) -> Dict[str, torch.Tensor]:
         """The inverse of load_state (checkpoint names, host tensors): what tests and tools hand to an independent implementation."""
         out = {"embed": self.embed, "final.norm": self.final_norm}
         if self.pre_norm:
             out["embed.norm"], out["head"] = self.embed_norm, self.head
+        if self.parallel:
+            out["head"] = self.head
+            if self.pair_table is not None:
+                out["bigram"] = self.pair_table
         for i, L in enumerate(self.layers):
             s, p = L.spec, f"l{i}.mix."
             H, d, dv = s.heads, s.dim, s.vdim
             out[f"l{i}.norm1"] = L.norm1
             if L.depth_w is not None:
                 out[f"l{i}.dwa"] = L.depth_w
-            if s.kind == "attention":
+            if self.parallel:
+                out[f"l{i}.ls1"] = L.ls1
+                if s.mlp is not None:
+                    out[f"l{i}.ls2"] = L.ls2
+                if L.shift is not None:
+                    out[f"l{i}.shift"] = L.shift
+            if L.sink is not None:
+                out[p + "sink"] = L.sink
+            if s.kind == "parallel":
+                a, b = p + "left.", p + "right."
+                G, sp = s.left.kv_heads, s.right
+                cuts = [H * d, G * d, G * dv]
+                out[a + "q"], out[a + "k"], out[a + "v"], out[b + "in"] = torch.split(L.w_in, cuts + [L.w_in.shape[0] - sum(cuts)], dim=0)
+                out[a + "q.b"], out[a + "k.b"], out[a + "v.b"] = torch.split(L.in_bias, cuts, dim=0)
+                out[a + "pb"], out[b + "conv"], out[b + "conv.b"], out[b + "dt_bias"] = L.pb, L.taps, L.conv_b, L.dt_bias
+                out[b + "A_log"], out[b + "D"], out[b + "norm"] = torch.log(-L.rate), L.skip, L.out_norm
+                out[a + "o"], out[b + "o"] = L.o[:, : H * dv], L.o[:, H * dv:]
+                out[a + "o.b"] = L.out_bias
+            elif s.kind == "attention":
                 cuts = [H * d, s.kv_heads * d, s.kv_heads * dv, H]
                 out[p + "q"], out[p + "k"], out[p + "v"], out[p + "g"] = torch.split(L.w_in, cuts, dim=0)
                 out[p + "talk"], out[p + "vmix"] = L.talk, L.lam.reshape(())
@@ -430,12 +620,15 @@ class HybridDecoder:
                 a, b = H * d, H * dv
                 out[p + "q"], out[p + "k"], out[p + "v"], out[p + "g"] = L.w_in[:a], L.w_in[a:2 * a], L.w_in[2 * a:2 * a + b], L.w_in[2 * a + b:]
                 out[p + "norm"] = L.out_norm
-            out[p + "o"] = L.o
+            if s.kind != "parallel":
+                out[p + "o"] = L.o
             if s.mlp is None and L.norm2 is not None:
                 out[f"l{i}.norm2"] = L.norm2
             if isinstance(s.mlp, DenseFfSpec):
                 q = f"l{i}.mlp."
-                out[f"l{i}.norm2"], out[q + "up"], out[q + "down"], out[q + "act"] = L.norm2, L.up, L.down, L.act
+                out[q + "up"], out[q + "down"], out[q + "act"] = L.up, L.down, L.act
+                if L.norm2 is not None:
+                    out[f"l{i}.norm2"] = L.norm2
             elif isinstance(s.mlp, MoeSpec) and s.mlp.gated:
                 q = f"l{i}.mlp."
                 out[f"l{i}.norm2"], out[q + "router"], out[q + "router.b"] = L.norm2, L.router, L.bias
@@ -462,14 +655,14 @@ class HybridDecoder:
         rows = kv.latent_rows(i)
         own = s.kv_from is None
         mixops.latent_prep(proj, q_abs, rows if own else None, batch.out_loc if own else None, batch.positions, L.cos_sin,
-                           L.c_norm, self.cfg.rms_norm_eps, H, d, r, R)
+                           L.c_norm, self.cfg.rms_norm_eps, H, d, r, R, interleaved=s.interleaved)
         mixops.gemm_nt(q_abs, proj, L.uk_t, T, R, d, lda=proj.stride(0), ldb=d, ldc=H * (R + r), groups=H, a_gs=d + r,
                        b_gs=R * d, c_gs=R + r)
         o_lat = torch.empty((T, H, R), dtype=torch.float32, device=h.device)
         # few query rows per request (decode, short portions): cut the keys into ranges so that the launch fills the chip
         splits = mixops.latent_attn_splits(md.batch, T, H, md.max_seqlen_k) if md.max_seqlen_q <= 16 else 1
         mixops.latent_attn(o_lat, q_abs, rows, ctx.page_table, md.req_rows, md.seq_lens, md.cu_seqlens_q, md.batch, R, s.scale,
-                           splits=splits)
+                           splits=splits, sink=L.sink)
         o = torch.empty((T, H * dv), dtype=self.dtype, device=h.device)
         mixops.gemm_nt(o, o_lat, L.uv, T, dv, R, lda=H * R, ldb=R, ldc=H * dv, groups=H, a_gs=R, b_gs=dv * R, c_gs=dv)
         return mixops.linear(o, L.o)
@@ -547,6 +740,75 @@ class HybridDecoder:
         mixops.gemm_nt(y, act, L.down, n, W, m.ff, lda=m.ff, ldb=m.ff, ldc=W, groups=m.experts, b_gs=W * m.ff, seg=seg, c_rows=perm)
         return y
 
+    def _pair(self, i: int, L: _Layer, g: torch.Tensor, ctx: Any, batch: Any) -> torch.Tensor:
+        """Sigmoid attention and a state-space layer on the same input: one input projection, the two mixers' kernels writing
+        their (scaled) outputs side by side into one row, one output projection."""
+        s, md, kv, eps = L.spec, batch.attn_metadata, ctx.kv_cache, self.cfg.rms_norm_eps
+        a, b = s.left, s.right
+        T, H, G, d, dv = g.shape[0], a.heads, a.kv_heads, a.dim, a.vdim
+        Hs, Gs, N, P = b.heads, b.kv_heads, b.dim, b.vdim
+        n_left, inner, C = (H + G) * d + G * dv, Hs * P, Hs * P + 2 * Gs * N
+        proj = mixops.linear(g, L.w_in)
+        cat = torch.empty((T, H * dv + inner), dtype=self.dtype, device=g.device)
+        # left: q / k prepared (bias, rotation, unit RMS), k and v into the cache rows, weights without normalisation over keys
+        kc, vc = kv.kv_rows(i)
+        q = mixops.qk_prep(proj, L.in_bias, kc, vc, batch.out_loc, batch.positions, L.cos_sin, eps, H, G, d, dv,
+                           interleaved=a.interleaved, unit=True)
+        mixops.sigmoid_attn(cat[:, : H * dv], q, kc, vc, ctx.page_table, md.req_rows, md.seq_lens, md.cu_seqlens_q, md.batch, H, G, d, dv,
+                            a.scale, a.softcap, L.pb, out_scale=s.left_scale,
+                            splits=mixops.sigmoid_attn_splits(md.batch, T, md.max_seqlen_k))
+        # right: proj[:, n_left:] = z | x B C | dt
+        z, xbc_raw, dt_raw = proj[:, n_left: n_left + inner], proj[:, n_left + inner: n_left + inner + C], proj[:, n_left + inner + C:]
+        xbc = mixops.short_conv(xbc_raw, C, L.taps, kv.conv_state(i), md.cu_seqlens_q, md.seq_lens, md.req_rows, md.batch,
+                                unit_heads=0, scaled_heads=0, d=1, bias=L.conv_b)
+        y = torch.empty((T, inner), dtype=torch.float32, device=g.device)
+        mixops.ssd(y, xbc, dt_raw, kv.state(i), L.rate, L.dt_bias, L.skip, md.cu_seqlens_q, md.seq_lens, md.req_rows, md.batch, Gs,
+                   chunks=getattr(md, "ssd_chunks", None))
+        mixops.gate_group_norm(cat[:, H * dv:], y, z, L.out_norm, eps, b.norm_groups, out_scale=s.right_scale)
+        return mixops.linear(cat, L.o)
+
+    def _forward_parallel(self, ctx: Any, batch: Any, layer_outputs: Optional[list]) -> torch.Tensor:
+        """One norm per layer, token-shifted mixer and feed-forward side by side -> the final-normed rows [tokens, W]."""
+        cfg, eps, md, kv = self.cfg, self.cfg.rms_norm_eps, batch.attn_metadata, ctx.kv_cache
+        T, W, n, dev, bs = batch.input_ids.shape[0], cfg.hidden_size, len(self.layers), self.device, batch.attn_metadata.batch
+        req = dict(positions=batch.positions, cu_q=md.cu_seqlens_q, req_rows=md.req_rows, batch=bs)
+        pe = cfg.pair_embed
+        x = mixops.embed_scaled(self.embed, batch.input_ids, cfg.embed_scale, pair=self.pair_table, buckets=pe[0] if pe else 0,
+                                mul_prev=pe[1] if pe else 0, mul_cur=pe[2] if pe else 0, prev_tok=kv.prev_token if pe else None, **req)
+        staging = torch.empty((n, bs, W), dtype=torch.float32, device=dev) if cfg.token_shift else None
+        hf = torch.empty((T, W), dtype=self.dtype, device=dev)
+
+        def open_layer(i: int, x_in: torch.Tensor, parts=(), bias=None, x_out=None):
+            """Closes the layer before (its parts summed onto x_in -> x_out) and opens layer i: -> (h, g)."""
+            if i == n:
+                mixops.shift_norm(x_in, self.final_norm, eps, dtype=self.dtype, w_offset=1.0, parts=parts, bias=bias, x_out=x_out, h_out=hf)
+                return hf, hf
+            L = self.layers[i]
+            h = torch.empty((T, W), dtype=self.dtype, device=dev) if L.spec.mlp is not None or L.shift is None else None
+            if L.shift is None:
+                mixops.shift_norm(x_in, L.norm1, eps, dtype=self.dtype, w_offset=1.0, parts=parts, bias=bias, x_out=x_out, h_out=h)
+                return h, h
+            g = torch.empty((T, W), dtype=self.dtype, device=dev)
+            mixops.shift_norm(x_in, L.norm1, eps, dtype=self.dtype, w_offset=1.0, parts=parts, bias=bias, x_out=x_out, h_out=h, g_out=g,
+                              shift=L.shift, state=kv.shift_state(i), staging=staging[i], **req)
+            return h, g
+
+        h, g = open_layer(0, x)
+        for i, L in enumerate(self.layers):
+            y = self._pair(i, L, g, ctx, batch) if L.spec.kind == "parallel" else self._latent(i, L, g, ctx, batch)
+            parts = [(y, L.ls1)]
+            if L.spec.mlp is not None:
+                parts.append((mixops.linear(mixops.xielu(mixops.linear(h, L.up), L.act), L.down), L.ls2))
+            x_next = torch.empty((T, W), dtype=torch.float32, device=dev)
+            h, g = open_layer(i + 1, x, parts, L.sum_bias, x_next)
+            x = x_next
+            if layer_outputs is not None:
+                layer_outputs.append(x.clone())
+        if cfg.token_shift or pe:
+            mixops.commit_rows(kv.shift_states if cfg.token_shift else None, staging, md.req_rows, bs, md.cu_seqlens_q,
+                               prev_tok=kv.prev_token if pe else None, ids=batch.input_ids if pe else None)
+        return hf
+
     def _forward_pre_norm(self, ctx: Any, batch: Any, layer_outputs: Optional[list]) -> torch.Tensor:
         """The pre-norm, depth-averaged stream -> the final-normed rows [tokens, W] in the model dtype."""
         cfg, eps = self.cfg, self.cfg.rms_norm_eps
@@ -594,8 +856,8 @@ class HybridDecoder:
         last token (prefill) or at every token (decode)."""
         cfg = self.cfg
         eps, alpha = cfg.rms_norm_eps, cfg.postln_alpha
-        if self.pre_norm:
-            hf = self._forward_pre_norm(ctx, batch, layer_outputs)
+        if self.pre_norm or self.parallel:
+            hf = self._forward_pre_norm(ctx, batch, layer_outputs) if self.pre_norm else self._forward_parallel(ctx, batch, layer_outputs)
             rows = getattr(batch, "logit_rows", None)
             if rows is None and batch.is_prefill:
                 rows = batch.attn_metadata.get_last_indices(batch.size)

@@ -80,7 +80,9 @@ def create_kvcache_pool(model_config, num_pages: int, page_size: int, dtype: tor
     """P/kvcache/__init__.py:27-44; a configuration that lists its layers one by one (`layers` of specs) gets the per-layer
     HybridCache with `state_rows` recurrent-state slots."""
     if hasattr(model_config, "layers"):
-        return HybridCache(model_config.layers, num_pages, page_size, state_rows, dtype, device)
+        return HybridCache(model_config.layers, num_pages, page_size, state_rows, dtype, device,
+                           shift_width=model_config.hidden_size if getattr(model_config, "token_shift", False) else 0,
+                           prev_token=getattr(model_config, "pair_embed", None) is not None)
     return MHAKVCache(num_kv_heads=model_config.num_kv_heads, num_pages=num_pages, page_size=page_size,
                       num_layers=model_config.num_layers, head_dim=model_config.head_dim, device=device,
                       dtype=dtype, tp_size=tp_size)
@@ -101,14 +103,32 @@ class HybridCache:
     * a delta-rule layer (`delta`, `channel_delta`) keeps the fp32 state `[heads, dim, vdim]` like a lightning layer and,
       beside it, the last `conv - 1` inputs of its short convolution: `conv_state(layer)` is `[state_rows, conv - 1,
       channels]` in the model dtype, channels = 2 * kv_heads * dim + heads * vdim, same row index.
-    Layers may differ in every size, so each gets its own allocation.
+    * a `parallel` layer (sigmoid attention beside a state-space layer) has both: `kv_rows(layer)` for the attention's keys and
+      values, `state(layer)` = fp32 `[state_rows, heads, state, vdim]` and `conv_state(layer)` = `[state_rows, conv - 1, heads *
+      vdim + 2 * groups * state]` for the state-space layer;
+    * a model whose mixers read a blend of a token's normed row and the previous token's (`shift_width` > 0) keeps, per layer and
+      request, the last normed row in fp32: `shift_state(layer)` is `[state_rows, width]` (all layers: `shift_states`);
+    * a model whose embedding depends on the previous token (`prev_token`) keeps each request's last token id: `prev_token`,
+      int32 `[state_rows]`.
+    Layers may differ in every size, so each gets its own allocation.  Every per-request row is indexed by the request's
+    page-table row and needs no clearing: a request whose first token is at position 0 never reads what the row held.
     """
 
-    def __init__(self, layers, num_pages: int, page_size: int, state_rows: int, dtype: torch.dtype, device: torch.device) -> None:
+    def __init__(self, layers, num_pages: int, page_size: int, state_rows: int, dtype: torch.dtype, device: torch.device,
+                 shift_width: int = 0, prev_token: bool = False) -> None:
         self._latent, self._state, self._owner, self._kv, self._conv = {}, {}, {}, {}, {}
         slots = num_pages * page_size
+        self.shift_states = torch.zeros((len(layers), state_rows, shift_width), dtype=torch.float32, device=device) if shift_width else None
+        self.prev_token = torch.zeros((state_rows,), dtype=torch.int32, device=device) if prev_token else None
         for i, spec in enumerate(layers):
-            if spec.kind == "latent_attention":
+            if spec.kind == "parallel":
+                a, b = spec.left, spec.right
+                self._kv[i] = (torch.zeros((slots, a.kv_heads * a.dim), dtype=dtype, device=device),
+                               torch.zeros((slots, a.kv_heads * a.vdim), dtype=dtype, device=device))
+                self._state[i] = torch.zeros((state_rows, b.heads, b.dim, b.vdim), dtype=torch.float32, device=device)
+                if b.conv > 1:
+                    self._conv[i] = torch.zeros((state_rows, b.conv - 1, b.heads * b.vdim + 2 * b.kv_heads * b.dim), dtype=dtype, device=device)
+            elif spec.kind == "latent_attention":
                 if spec.kv_from is None:
                     self._latent[i] = torch.zeros((slots, spec.kv_rank + spec.rot_dim), dtype=dtype, device=device)
                 self._owner[i] = i if spec.kv_from is None else spec.kv_from
@@ -143,22 +163,30 @@ class HybridCache:
         return self._kv[layer]
 
     def conv_state(self, layer: int):
-        """[state_rows, conv - 1, channels] of a delta-rule layer, or None when its convolution has one tap."""
+        """[state_rows, conv - 1, channels] of a delta-rule or state-space layer, or None when its convolution has one tap."""
         return self._conv.get(layer)
+
+    def shift_state(self, layer: int) -> torch.Tensor:
+        """fp32 [state_rows, width]: every request's last normed row of this layer."""
+        return self.shift_states[layer]
 
     @staticmethod
     def bytes_per_page(layers, page_size: int, dtype: torch.dtype) -> int:
         es = torch.empty((), dtype=dtype).element_size()
         per_token = sum(s.kv_rank + s.rot_dim for s in layers if s.kind == "latent_attention" and s.kv_from is None)
         per_token += sum(s.kv_heads * (s.dim + s.vdim) for s in layers if s.kind == "attention")
+        per_token += sum(s.left.kv_heads * (s.left.dim + s.left.vdim) for s in layers if s.kind == "parallel")
         return per_token * es * page_size
 
     @staticmethod
-    def state_bytes(layers, state_rows: int, dtype: torch.dtype = torch.bfloat16) -> int:
+    def state_bytes(layers, state_rows: int, dtype: torch.dtype = torch.bfloat16, shift_width: int = 0) -> int:
         es = torch.empty((), dtype=dtype).element_size()
         total = sum(4 * s.heads * s.dim * s.vdim * state_rows for s in layers if s.kind in ("lightning", "delta", "channel_delta"))
-        return total + sum(es * (s.conv - 1) * (2 * s.kv_heads * s.dim + s.heads * s.vdim) * state_rows
-                           for s in layers if s.kind in ("delta", "channel_delta"))
+        total += sum(es * (s.conv - 1) * (2 * s.kv_heads * s.dim + s.heads * s.vdim) * state_rows
+                     for s in layers if s.kind in ("delta", "channel_delta"))
+        for s in (x.right for x in layers if x.kind == "parallel"):
+            total += (4 * s.heads * s.dim * s.vdim + es * (s.conv - 1) * (s.heads * s.vdim + 2 * s.kv_heads * s.dim)) * state_rows
+        return total + 4 * shift_width * len(layers) * state_rows
 
     @property
     def device(self) -> torch.device:

@@ -91,8 +91,9 @@ def postnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, *, y: Optional[t
 
 def latent_prep(proj: torch.Tensor, q_abs: torch.Tensor, cache: Optional[torch.Tensor], out_loc: Optional[torch.Tensor],
                 positions: torch.Tensor, cos_sin: torch.Tensor, c_norm_w: Optional[torch.Tensor], eps: float, H: int, d: int,
-                r: int, R: int) -> None:
-    """Rotates the query parts into q_abs[:, :, R:]; with `cache`, norms + rotates + stores this layer's own latent rows."""
+                r: int, R: int, interleaved: bool = False) -> None:
+    """Rotates the query parts into q_abs[:, :, R:]; with `cache`, norms + rotates + stores this layer's own latent rows.
+    interleaved: entries (2i, 2i + 1) of a rotated part form pair i instead of (i, i + half)."""
     _dev(proj, q_abs, cache, out_loc, positions, cos_sin, c_norm_w)
     T = proj.shape[0]
     has_kv = cache is not None
@@ -105,7 +106,7 @@ def latent_prep(proj: torch.Tensor, q_abs: torch.Tensor, cache: Optional[torch.T
     check_mix(mix_lib().msgl_mix_latent_prep(
         proj.data_ptr(), proj.stride(0), q_abs.data_ptr(), _p(cache), _p(None if out_loc is None else _i32(out_loc)),
         _i32(positions).data_ptr(), cos_sin.data_ptr(), _p(c_norm_w), float(eps), T, H, d, r, cos_sin.shape[1], R, int(has_kv),
-        _code(proj), _stream()), "latent_prep")
+        int(interleaved), _code(proj), _stream()), "latent_prep")
 
 
 def latent_attn_splits(batch: int, total_q: int, H: int, max_keys: int) -> int:
@@ -118,8 +119,11 @@ def latent_attn_splits(batch: int, total_q: int, H: int, max_keys: int) -> int:
 
 
 def latent_attn(out: torch.Tensor, q_abs: torch.Tensor, cache: torch.Tensor, table: torch.Tensor, req_rows: torch.Tensor,
-                seq_lens: torch.Tensor, cu_q: torch.Tensor, batch: int, dv: int, scale: float, splits: int = 1) -> None:
-    _dev(out, q_abs, cache, table, req_rows, seq_lens, cu_q)
+                seq_lens: torch.Tensor, cu_q: torch.Tensor, batch: int, dv: int, scale: float, splits: int = 1,
+                sink: Optional[torch.Tensor] = None) -> None:
+    """sink (fp32 [H]): one more term exp(sink[h]) in every softmax denominator of head h, with no key and no value."""
+    _dev(out, q_abs, cache, table, req_rows, seq_lens, cu_q, sink)
+    assert sink is None or (sink.dtype == torch.float32 and sink.is_contiguous() and sink.shape == (q_abs.shape[1],))
     T, H, dk = q_abs.shape
     assert q_abs.dtype == torch.float32 and q_abs.is_contiguous() and out.dtype == torch.float32 and out.is_contiguous()
     assert out.shape == (T, H, dv) and cache.is_contiguous() and cache.shape[1] == dk
@@ -130,7 +134,7 @@ def latent_attn(out: torch.Tensor, q_abs: torch.Tensor, cache: torch.Tensor, tab
         ws = torch.empty(mix_lib().msgl_mix_latent_attn_workspace_floats(T, H, dv, splits), dtype=torch.float32, device=out.device)
     check_mix(mix_lib().msgl_mix_latent_attn(
         out.data_ptr(), q_abs.data_ptr(), cache.data_ptr(), table.data_ptr(), table.stride(0), _i32(req_rows).data_ptr(),
-        _i32(seq_lens).data_ptr(), _i32(cu_q).data_ptr(), batch, T, H, dk, dv, float(scale), _code(cache), splits, _p(ws),
+        _i32(seq_lens).data_ptr(), _i32(cu_q).data_ptr(), batch, T, H, dk, dv, float(scale), _p(sink), _code(cache), splits, _p(ws),
         _stream()), "latent_attn")
 
 
@@ -383,16 +387,17 @@ def window_attn(out: torch.Tensor, src: torch.Tensor, g_off: int, k_cache: torch
 
 
 def short_conv(src: torch.Tensor, C: int, taps: torch.Tensor, state: Optional[torch.Tensor], cu_q: torch.Tensor, seq_lens: torch.Tensor,
-               slots: torch.Tensor, batch: int, unit_heads: int, scaled_heads: int, d: int) -> torch.Tensor:
+               slots: torch.Tensor, batch: int, unit_heads: int, scaled_heads: int, d: int, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal per-channel convolution + SiLU of src[:, :C] (taps [C, n]; state [slots, n - 1, C] carries the inputs before the
     portion and is moved on), unit vectors for the first `unit_heads` groups of d channels -> fp32 [T, C]."""
-    _dev(src, taps, state, cu_q, seq_lens, slots)
+    _dev(src, taps, state, cu_q, seq_lens, slots, bias)
     T, n = src.shape[0], taps.shape[1]
+    assert bias is None or (bias.dtype == src.dtype and bias.shape == (C,) and bias.is_contiguous())
     assert src.stride(1) == 1 and taps.is_contiguous() and taps.shape[0] == C and taps.dtype == src.dtype
     assert n == 1 or (state.is_contiguous() and state.dtype == src.dtype and state.shape[1:] == (n - 1, C))
     out = torch.empty((T, C), dtype=torch.float32, device=src.device)
     check_mix(mix_lib().msgl_mix_short_conv(
-        out.data_ptr(), src.data_ptr(), src.stride(0), taps.data_ptr(), _p(state), _i32(cu_q).data_ptr(), _i32(seq_lens).data_ptr(),
+        out.data_ptr(), src.data_ptr(), src.stride(0), taps.data_ptr(), _p(bias), _p(state), _i32(cu_q).data_ptr(), _i32(seq_lens).data_ptr(),
         _i32(slots).data_ptr(), batch, T, C, n, unit_heads, scaled_heads, d, _code(src), _stream()), "short_conv")
     return out
 
@@ -434,4 +439,169 @@ def head_gated_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, e
     out = torch.empty((rows, H * dv), dtype=gate.dtype, device=o.device)
     check_mix(mix_lib().msgl_mix_head_gated_norm(out.data_ptr(), o.data_ptr(), gate.data_ptr(), gate.stride(0), weight.data_ptr(),
                                                  float(eps), rows, H, dv, gate_act, _code(gate), _stream()), "head_gated_norm")
+    return out
+
+
+# ------------------------------------------------------------------ parallel-residual hybrid decoders (csrc/mix_par.hip)
+def _f32(t: Optional[torch.Tensor], n: int) -> Optional[torch.Tensor]:
+    assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.shape == (n,)), (None if t is None else (t.dtype, t.shape))
+    return t
+
+
+def embed_scaled(table: torch.Tensor, ids: torch.Tensor, scale: float, out: Optional[torch.Tensor] = None, *, pair: Optional[torch.Tensor] = None,
+                 buckets: int = 0, mul_prev: int = 0, mul_cur: int = 0, positions: Optional[torch.Tensor] = None,
+                 cu_q: Optional[torch.Tensor] = None, req_rows: Optional[torch.Tensor] = None, batch: int = 0,
+                 prev_tok: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """-> fp32 [T, W] = scale * table[id] + pair[(previous id * mul_prev + id * mul_cur) mod buckets] (pair row `buckets` at position
+    0; the id before a portion's first token: prev_tok[req_rows[b]], int32)."""
+    _dev(table, ids, pair, positions, cu_q, req_rows, prev_tok)
+    T, W = ids.shape[0], table.shape[1]
+    assert table.is_contiguous() and (pair is None or (pair.is_contiguous() and pair.dtype == table.dtype and pair.shape == (buckets + 1, W)))
+    if out is None:
+        out = torch.empty((T, W), dtype=torch.float32, device=table.device)
+    assert out.dtype == torch.float32 and out.is_contiguous() and out.shape == (T, W)
+    check_mix(mix_lib().msgl_mix_embed_scaled(
+        out.data_ptr(), table.data_ptr(), _p(pair), _i32(ids).data_ptr(), _p(positions), _p(cu_q), _p(req_rows), batch, _p(prev_tok),
+        float(scale), buckets, mul_prev, mul_cur, T, W, _code(table), _stream()), "embed_scaled")
+    return out
+
+
+def shift_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, *, dtype: torch.dtype, w_offset: float = 0.0, parts=(), bias: Optional[torch.Tensor] = None,
+               x_out: Optional[torch.Tensor] = None, h_out: Optional[torch.Tensor] = None, g_out: Optional[torch.Tensor] = None,
+               shift: Optional[torch.Tensor] = None, state: Optional[torch.Tensor] = None, staging: Optional[torch.Tensor] = None,
+               positions: Optional[torch.Tensor] = None, cu_q: Optional[torch.Tensor] = None, req_rows: Optional[torch.Tensor] = None,
+               batch: int = 0) -> None:
+    """row = x + bias + sum over parts (y, v) of v * y -> x_out (fp32; a buffer other than x);  h = rms_unit(row) * (weight + w_offset) -> h_out;
+    with `shift`: g = h + (h of the token before - h) * shift -> g_out (the token before a portion: state[req_rows[b]], fp32; the
+    last h of request b -> staging[b]).  weight, shift, bias and the v of a part: fp32 [W]; y: [rows, W] views in `dtype`."""
+    rows, W = x.shape
+    _dev(x, weight, bias, x_out, h_out, g_out, shift, state, staging, positions, cu_q, req_rows)
+    assert x.dtype == torch.float32 and x.is_contiguous() and len(parts) <= 2
+    _f32(weight, W), _f32(bias, W), _f32(shift, W)
+    ys = []
+    for y, v in parts:
+        _dev(y, v)
+        assert y.dtype == dtype and y.shape == (rows, W) and y.stride(1) == 1
+        ys.append((y.data_ptr(), y.stride(0), _p(_f32(v, W))))
+    ys += [(0, 0, 0)] * (2 - len(ys))
+    for o, dt in ((x_out, torch.float32), (h_out, dtype), (g_out, dtype)):
+        assert o is None or (o.shape == (rows, W) and o.is_contiguous() and o.dtype == dt)
+    if shift is not None:
+        assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1] == W
+        assert staging.dtype == torch.float32 and staging.is_contiguous() and staging.shape == (batch, W)
+    if rows:
+        check_mix(mix_lib().msgl_mix_shift_norm(
+            x.data_ptr(), _p(x_out), ys[0][0], ys[0][1], ys[0][2], ys[1][0], ys[1][1], ys[1][2], _p(bias), weight.data_ptr(), float(w_offset), _p(shift),
+            _p(h_out), _p(g_out), _p(state), _p(staging), _p(positions), _p(cu_q), _p(req_rows), batch, float(eps), rows, W,
+            _lib.BF16 if dtype == torch.bfloat16 else _lib.F32, _stream()), "shift_norm")
+
+
+def commit_rows(dst: Optional[torch.Tensor], src: Optional[torch.Tensor], slots: torch.Tensor, batch: int, cu_q: torch.Tensor,
+                prev_tok: Optional[torch.Tensor] = None, ids: Optional[torch.Tensor] = None) -> None:
+    """dst[l, slots[b]] = src[l, b] (fp32 [L, rows, W] <- [L, batch, W]); prev_tok[slots[b]] = the last id of request b."""
+    _dev(dst, src, slots, cu_q, prev_tok, ids)
+    L = W = 0
+    if dst is not None:
+        L, _, W = dst.shape
+        assert dst.dtype == torch.float32 and dst.is_contiguous() and src.dtype == torch.float32 and src.is_contiguous()
+        assert src.shape == (L, batch, W)
+    check_mix(mix_lib().msgl_mix_commit_rows(_p(dst), 0 if dst is None else dst.stride(0), _p(src), 0 if src is None else src.stride(0), L,
+                                             _i32(slots).data_ptr(), batch, W, _p(prev_tok), _p(ids), _i32(cu_q).data_ptr(), _stream()),
+              "commit_rows")
+
+
+def qk_prep(proj: torch.Tensor, bias: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: torch.Tensor, out_loc: torch.Tensor,
+            positions: torch.Tensor, cos_sin: Optional[torch.Tensor], eps: float, H: int, G: int, d: int, dv: int, *, interleaved: bool,
+            unit: bool) -> torch.Tensor:
+    """Projection rows [q | k | v | ...] (+ fp32 bias) -> rotated (and unit-RMS) q as fp32 [T, H * d]; k, v into the cache rows."""
+    _dev(proj, bias, k_cache, v_cache, out_loc, positions, cos_sin)
+    T = proj.shape[0]
+    n = (H + G) * d + G * dv
+    assert proj.stride(1) == 1 and proj.shape[1] >= n and (bias is None or _f32(bias, n) is not None)
+    assert k_cache.is_contiguous() and k_cache.shape[1] == G * d and v_cache.is_contiguous() and v_cache.shape[1] == G * dv
+    assert k_cache.dtype == proj.dtype == v_cache.dtype and out_loc.shape[0] == T
+    rd = 0
+    if cos_sin is not None:
+        assert cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.dim() == 2
+        rd = cos_sin.shape[1]
+    q = torch.empty((T, H * d), dtype=torch.float32, device=proj.device)
+    check_mix(mix_lib().msgl_mix_qk_prep(
+        proj.data_ptr(), proj.stride(0), _p(bias), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _i32(out_loc).data_ptr(),
+        _i32(positions).data_ptr(), _p(cos_sin), rd, int(interleaved), int(unit), float(eps), T, H, G, d, dv, _code(proj), _stream()),
+        "qk_prep")
+    return q
+
+
+def sigmoid_attn_splits(batch: int, total_q: int, max_keys: int) -> int:
+    """Key ranges per request for a step with few query tokens: enough workgroups to fill the chip, at least 256 keys each.  A
+    function of static sizes only, so a captured graph keeps its grid."""
+    if total_q >= 8 * batch and total_q >= 256:
+        return 1
+    return max(1, min(512 // max(total_q + batch, 1), max_keys // 256, 32))
+
+
+def sigmoid_attn(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, table: torch.Tensor, req_rows: torch.Tensor,
+                 seq_lens: torch.Tensor, cu_q: torch.Tensor, batch: int, H: int, G: int, d: int, dv: int, scale: float, softcap: float,
+                 pb: Optional[torch.Tensor], out_scale: float = 1.0, splits: int = 1) -> None:
+    """out[:, : H * dv] (a view with a row stride is fine) = out_scale * sum over visible keys of sigmoid(cap(scale q.k) + pb[h]) v."""
+    _dev(out, q, k_cache, v_cache, table, req_rows, seq_lens, cu_q, pb)
+    T = q.shape[0]
+    assert q.dtype == torch.float32 and q.is_contiguous() and q.shape == (T, H * d)
+    assert out.shape == (T, H * dv) and out.stride(1) == 1 and out.dtype == k_cache.dtype == v_cache.dtype
+    assert k_cache.is_contiguous() and k_cache.shape[1] == G * d and v_cache.is_contiguous() and v_cache.shape[1] == G * dv
+    assert table.dtype == torch.int32 and table.stride(1) == 1 and (pb is None or _f32(pb, H) is not None)
+    assert req_rows.numel() >= batch and seq_lens.numel() >= batch and cu_q.numel() >= batch + 1
+    ws = None
+    if splits > 1:
+        ws = torch.empty(mix_lib().msgl_mix_sigmoid_attn_workspace_floats(T, H, dv, splits), dtype=torch.float32, device=out.device)
+    check_mix(mix_lib().msgl_mix_sigmoid_attn(
+        out.data_ptr(), out.stride(0), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), table.data_ptr(), table.stride(0),
+        _i32(req_rows).data_ptr(), _i32(seq_lens).data_ptr(), _i32(cu_q).data_ptr(), batch, T, H, G, d, dv, float(scale), float(softcap),
+        _p(pb), float(out_scale), _code(k_cache), splits, _p(ws), _stream()), "sigmoid_attn")
+
+
+def ssd(out: torch.Tensor, xbc: torch.Tensor, dt_raw: torch.Tensor, state: torch.Tensor, rate: torch.Tensor, dt_bias: torch.Tensor,
+        D: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor, slots: torch.Tensor, batch: int, G: int, chunks=None) -> None:
+    """state: fp32 [slots, H, N, P]; xbc: fp32 rows [x H*P | B G*N | C G*N]; dt_raw [T, H] in the model dtype (a view with a row
+    stride is fine); rate = -exp(A_log), dt_bias, D in fp32 [H].  chunks = (items int32 [n, 3], item_first int32 [batch + 1], n)
+    cuts long portions into pieces that run in parallel."""
+    _dev(out, xbc, dt_raw, state, rate, dt_bias, D, cu_q, seq_lens, slots)
+    _, H, N, P = state.shape
+    T = xbc.shape[0]
+    assert state.dtype == torch.float32 and state.is_contiguous() and xbc.dtype == torch.float32 and xbc.stride(1) == 1
+    assert xbc.shape[1] == H * P + 2 * G * N and out.dtype == torch.float32 and out.is_contiguous() and out.shape == (T, H * P)
+    assert dt_raw.shape == (T, H) and dt_raw.stride(1) == 1
+    _f32(rate, H), _f32(dt_bias, H), _f32(D, H)
+    items = first = scratch = None
+    n_items = 0
+    if chunks is not None:
+        items, first, n_items = chunks
+        _dev(items, first)
+        assert items.numel() == 3 * n_items and first.numel() == batch + 1
+        scratch = torch.empty(n_items * H * (N * P + 1), dtype=torch.float32, device=out.device)
+    check_mix(mix_lib().msgl_mix_ssd(
+        out.data_ptr(), xbc.data_ptr(), xbc.stride(0), dt_raw.data_ptr(), dt_raw.stride(0), state.data_ptr(), rate.data_ptr(),
+        dt_bias.data_ptr(), D.data_ptr(), _i32(cu_q).data_ptr(), _i32(seq_lens).data_ptr(), _i32(slots).data_ptr(), batch, H, G, N, P,
+        _code(dt_raw), n_items, _p(None if items is None else _i32(items)), _p(None if first is None else _i32(first)), _p(scratch),
+        _stream()), "ssd")
+
+
+def gate_group_norm(out: torch.Tensor, y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float, groups: int,
+                    out_scale: float = 1.0) -> None:
+    """out (a [rows, N] view, model dtype) = rms_unit per group of (y * silu(z)) * weight * out_scale; y fp32, z a view in out's dtype."""
+    _dev(out, y, z, weight)
+    rows, N = y.shape
+    assert y.dtype == torch.float32 and y.is_contiguous() and z.shape == (rows, N) and z.stride(1) == 1 and z.dtype == out.dtype
+    assert out.shape == (rows, N) and out.stride(1) == 1 and _f32(weight, N) is not None
+    check_mix(mix_lib().msgl_mix_gate_group_norm(out.data_ptr(), out.stride(0), y.data_ptr(), z.data_ptr(), z.stride(0), weight.data_ptr(),
+                                                 float(eps), rows, N, groups, float(out_scale), _code(z), _stream()), "gate_group_norm")
+
+
+def xielu(z: torch.Tensor, pq: torch.Tensor) -> torch.Tensor:
+    """z > 0: softplus(p) z^2 + z / 2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2;  pq = (p, q) fp32 on the device."""
+    _dev(z, pq)
+    rows, N = z.shape
+    assert z.stride(1) == 1 and _f32(pq, 2) is not None
+    out = torch.empty((rows, N), dtype=z.dtype, device=z.device)
+    check_mix(mix_lib().msgl_mix_xielu(out.data_ptr(), z.data_ptr(), z.stride(0), pq.data_ptr(), rows, N, _code(z), _stream()), "xielu")
     return out
