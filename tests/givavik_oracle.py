@@ -84,6 +84,43 @@ def latent_rows(m: dict, st, p: str, g: torch.Tensor, eps: float):
     return c, kr
 
 
+def sink_softmax_rows(s: torch.Tensor, v: torch.Tensor, sink: float) -> torch.Tensor:
+    """One query: scores s [n] over its visible keys, values v [n, e]; the denominator holds one more term exp(sink)."""
+    top = max(float(s.max()), float(sink))
+    e = torch.exp(s - top)
+    return (e @ v) / (e.sum() + math.exp(float(sink) - top))
+
+
+def sigmoid_weighted_sum(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, pb: torch.Tensor, scale: float, cap: float) -> torch.Tensor:
+    """q [T, H, d], k [T, G, d], v [T, G, e] of one sequence -> [T, H, e]: every visible key weighs sigmoid(cap tanh(s / cap) + pb_h),
+    s = scale q.k, nothing is normalised (cap <= 0: no soft cap)."""
+    T, H, _ = q.shape
+    rep = H // k.shape[1]
+    out = torch.zeros(T, H, v.shape[-1], dtype=F64)
+    for h in range(H):
+        for i in range(T):
+            s = (k[: i + 1, h // rep] @ q[i, h]) * scale
+            if cap > 0:
+                s = cap * torch.tanh(s / cap)
+            out[i, h] = torch.sigmoid(s + pb[h]) @ v[: i + 1, h // rep]
+    return out
+
+
+def state_space_scan(xs: torch.Tensor, Bm: torch.Tensor, Cm: torch.Tensor, dt: torch.Tensor, A: torch.Tensor, D: torch.Tensor,
+                     S0: Optional[torch.Tensor] = None):
+    """xs [T, H, P], Bm / Cm [T, G, N], dt [T, H] (already positive), A [H] > 0, D [H] -> (y [T, H, P], final state [H, N, P])."""
+    T, H, P = xs.shape
+    G, N = Bm.shape[1], Bm.shape[2]
+    y = torch.zeros(T, H, P, dtype=F64)
+    S = torch.zeros(H, N, P, dtype=F64) if S0 is None else S0.clone()
+    for h in range(H):
+        gi = h // (H // G)
+        for t in range(T):
+            S[h] = torch.exp(-A[h] * dt[t, h]) * S[h] + dt[t, h] * torch.outer(Bm[t, gi], xs[t, h])
+            y[t, h] = S[h].T @ Cm[t, gi] + D[h] * xs[t, h]
+    return y, S
+
+
 def latent_attention(m: dict, st, p: str, g: torch.Tensor, c: torch.Tensor, kr: torch.Tensor) -> torch.Tensor:
     H, d, r, dv, R = int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), int(m["kv_rank"])
     T = g.shape[0]
@@ -96,9 +133,7 @@ def latent_attention(m: dict, st, p: str, g: torch.Tensor, c: torch.Tensor, kr: 
     for h in range(H):
         for i in range(T):
             s = (k[: i + 1, h] @ qn[i, h] + kr[: i + 1] @ qr[i, h]) * float(m["scale"])
-            top = max(float(s.max()), float(sink[h]))
-            e = torch.exp(s - top)
-            out[i, h] = (e @ v[: i + 1, h]) / (e.sum() + math.exp(float(sink[h]) - top))
+            out[i, h] = sink_softmax_rows(s, v[: i + 1, h], float(sink[h]))
     return out.reshape(T, H * dv) @ st[p + "o"].to(F64).T
 
 
@@ -107,18 +142,12 @@ def sigmoid_attention(m: dict, st, p: str, g: torch.Tensor, eps: float) -> torch
     T = g.shape[0]
     pos = torch.arange(T)
     lin = lambda n: g @ st[p + n].to(F64).T + st[p + n + ".b"].to(F64)
-    dims, base = int(m["rot"]["dims"]), float(m["rot"]["base"])
+    rot = m.get("rot") or {}
+    dims, base = int(rot.get("dims", 0)), float(rot.get("base", 10000.0))
     q = rms_unit(rotate_pairs(lin("q").view(T, H, d), pos, dims, base), eps)
     k = rms_unit(rotate_pairs(lin("k").view(T, G, d), pos, dims, base), eps)
     v = lin("v").view(T, G, dv)
-    cap, pb = float(m["softcap"]), st[p + "pb"].to(F64)
-    out = torch.zeros(T, H, dv, dtype=F64)
-    for h in range(H):
-        kh = h // (H // G)
-        for i in range(T):
-            s = (k[: i + 1, kh] @ q[i, h]) * float(m["scale"])
-            s = cap * torch.tanh(s / cap)
-            out[i, h] = torch.sigmoid(s + pb[h]) @ v[: i + 1, kh]
+    out = sigmoid_weighted_sum(q, k, v, st[p + "pb"].to(F64), float(m["scale"]), float(m.get("softcap") or 0.0))
     return out.reshape(T, H * dv) @ st[p + "o"].to(F64).T + st[p + "o.b"].to(F64)
 
 
@@ -138,13 +167,7 @@ def state_space(m: dict, st, p: str, g: torch.Tensor, eps: float) -> torch.Tenso
     Cm = conv[:, inner + G * N:].view(T, G, N)
     dt = softplus(dt + st[p + "dt_bias"].to(F64))
     A, D = torch.exp(st[p + "A_log"].to(F64)), st[p + "D"].to(F64)
-    y = torch.zeros(T, H, P, dtype=F64)
-    for h in range(H):
-        gi = h // (H // G)
-        S = torch.zeros(N, P, dtype=F64)
-        for t in range(T):
-            S = torch.exp(-A[h] * dt[t, h]) * S + dt[t, h] * torch.outer(Bm[t, gi], xs[t, h])
-            y[t, h] = S.T @ Cm[t, gi] + D[h] * xs[t, h]
+    y, _ = state_space_scan(xs, Bm, Cm, dt, A, D)
     y = y.reshape(T, inner) * silu(z)
     y = rms_unit(y.view(T, ng, inner // ng), eps).reshape(T, inner) * st[p + "norm"].to(F64)
     return y @ st[p + "o"].to(F64).T
