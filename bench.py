@@ -671,11 +671,21 @@ def main() -> None:
                          "attention with mixed heads + gated delta-rule layers) beside the post-norm hybrid decoder of equal size, "
                          "and its kernels against their rooflines (tools/bedarax_bench.py; further flags after --bedarax-args)")
     ap.add_argument("--bedarax-args", nargs=argparse.REMAINDER, default=[], help="flags handed to tools/bedarax_bench.py")
+    ap.add_argument("--givavik", action="store_true",
+                    help="instead of the default workload: prefill / decode throughput of the parallel-residual hybrid decoder (latent "
+                         "attention with a sink, sigmoid attention beside a state-space layer) beside the post-norm hybrid decoder of "
+                         "equal size, and its kernels against their rooflines (tools/givavik_bench.py; further flags after --givavik-args)")
+    ap.add_argument("--givavik-args", nargs=argparse.REMAINDER, default=[], help="flags handed to tools/givavik_bench.py")
     args = ap.parse_args()
     if args.bedarax:
         from tools.bedarax_bench import main as bedarax_main
 
         bedarax_main(list(args.bedarax_args))
+        return
+    if args.givavik:
+        from tools.givavik_bench import main as givavik_main
+
+        givavik_main(list(args.givavik_args))
         return
     if args.hybrid:
         from tools.hybrid_bench import main as hybrid_main
