@@ -1,4 +1,4 @@
-// Shared device helpers and host-side argument checks of the sequence-mixing kernels (seqmix.hip, seqmix2.hip).
+// Shared device helpers and host-side argument checks of the sequence-mixing kernels (seqmix.hip, mix_delta.hip, mix_par.hip).
 // Everything lives in an anonymous namespace: each translation unit of libmsgl_mix.so gets its own copy, and the one
 // per-thread error text is reached through msgl_mix_set_error / msgl_mix_last_error.
 #ifndef MSGL_MIX_COMMON_H_
@@ -91,6 +91,73 @@ const T* cp(const void* p) {
 template <typename T>
 T* mp(void* p) {
   return static_cast<T*>(p);
+}
+
+// ---- matrix-core helpers: fragment types, packed bf16 loads
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+struct __attribute__((aligned(16))) Q4 {
+  uint32_t x, y, z, w;
+};
+__device__ __forceinline__ uint32_t bf16_bits(float v) {
+  bf16_t t;
+  st(&t, v);
+  return t.bits;
+}
+
+// eight consecutive k of one row as packed bf16; `n` of them exist (the rest read as zero); vec: 16-byte loads are legal
+__device__ __forceinline__ Q4 load8(const bf16_t* p, int n, bool vec) {
+  if (vec && n >= 8) return *reinterpret_cast<const Q4*>(p);
+  uint32_t e[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) e[i] = i < n ? p[i].bits : 0u;
+  return Q4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+}
+__device__ __forceinline__ Q4 load8(const float* p, int n, bool vec) {
+  float f[8];
+  if (vec && n >= 8) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = i < n ? p[i] : 0.f;
+  }
+  return Q4{bf16_bits(f[0]) | (bf16_bits(f[1]) << 16), bf16_bits(f[2]) | (bf16_bits(f[3]) << 16),
+            bf16_bits(f[4]) | (bf16_bits(f[5]) << 16), bf16_bits(f[6]) | (bf16_bits(f[7]) << 16)};
+}
+
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((address_space(3))) s16x4_t lds_s16x4_t;
+
+// Which request and which of its QT-token groups workgroup `blockIdx.x` owns: group counts ceil(new tokens / QT) of up to 256
+// requests at a time, scanned by the whole workgroup (one pass of independent loads instead of one thread walking the batch).
+// Leaves request -1 for workgroups past the last group.  cnt: 256 ints of LDS; every thread of the (256-thread) workgroup calls.
+__device__ __forceinline__ void find_group(const int* __restrict__ cu_q, int B, int QT, int* cnt, int* s_req, int* s_tok0) {
+  const int tid = threadIdx.x;
+  if (tid == 0) *s_req = -1;
+  int base = 0;
+  for (int c0 = 0; c0 < B; c0 += 256) {
+    const int b = c0 + tid;
+    const int g = b < B ? (cu_q[b + 1] - cu_q[b] + QT - 1) / QT : 0;
+    cnt[tid] = g;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+      const int v = tid >= off ? cnt[tid - off] : 0;
+      __syncthreads();
+      cnt[tid] += v;
+      __syncthreads();
+    }
+    const int incl = cnt[tid], total = cnt[255];
+    const int target = (int)blockIdx.x - base;
+    if (b < B && target >= incl - g && target < incl) {
+      *s_req = b;
+      *s_tok0 = (target - (incl - g)) * QT;
+    }
+    __syncthreads();
+    if (target < total) break;
+    base += total;
+  }
+  __syncthreads();
 }
 
 bool dtype_ok(int dt) { return dt == MSGL_MIX_BF16 || dt == MSGL_MIX_F32; }

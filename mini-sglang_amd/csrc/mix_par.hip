@@ -12,8 +12,10 @@
 //                           previous row; first token of a portion: the request's state row; position 0: zero)
 //   commit_rows_kernel      after the forward: every request's last h of every layer -> its state row; its last token id
 //   qk_prep_kernel          q, k (+ bias), rotation of the leading entries of each head, unit-RMS q and k; k, v -> cache rows
-//   sigmoid_attn_kernel     o[t, h] = sum_{j <= t} sigmoid(cap(scale q . k_j) + b_h) v_j, no normalisation over keys; key ranges
-//                           are plain partial sums (sigmoid_merge_kernel adds them)
+//   sigmoid_attn_mfma_kernel  o[t, h] = sum_{j <= t} sigmoid(cap(scale q . k_j) + b_h) v_j, no normalisation over keys; bf16 caches,
+//                           both products on the matrix cores, weights in fp32; key ranges are plain partial sums
+//                           (sigmoid_merge_kernel adds them)
+//   sigmoid_attn_kernel     the same in plain fp32 (fp32 caches, heads past the matrix-core instances)
 //   ssd_kernel              S <- exp(rate dt) S + dt B x^T,  y = S^T C + D x per (request, head); a thread owns one column of S;
 //                           long portions as parallel chunks joined by ssd_scan_kernel
 //   gate_group_norm_kernel  (y * silu(z)) normed in equal groups of the row, times w
@@ -186,35 +188,6 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const T* __restrict__ proj
 constexpr int kSigRows = 16;
 constexpr int kSigMaxC = 16;  // value columns per lane: dv <= 256
 
-// defined in seqmix.hip's anonymous namespace as well; this unit keeps its own copy
-__device__ __forceinline__ void find_group(const int* __restrict__ cu_q, int B, int QT, int* cnt, int* s_req, int* s_tok0) {
-  const int tid = threadIdx.x;
-  if (tid == 0) *s_req = -1;
-  int base = 0;
-  for (int c0 = 0; c0 < B; c0 += 256) {
-    const int b = c0 + tid;
-    const int g = b < B ? (cu_q[b + 1] - cu_q[b] + QT - 1) / QT : 0;
-    cnt[tid] = g;
-    __syncthreads();
-    for (int off = 1; off < 256; off <<= 1) {
-      const int v = tid >= off ? cnt[tid - off] : 0;
-      __syncthreads();
-      cnt[tid] += v;
-      __syncthreads();
-    }
-    const int incl = cnt[tid], total = cnt[255];
-    const int target = (int)blockIdx.x - base;
-    if (b < B && target >= incl - g && target < incl) {
-      *s_req = b;
-      *s_tok0 = (target - (incl - g)) * QT;
-    }
-    __syncthreads();
-    if (target < total) break;
-    base += total;
-  }
-  __syncthreads();
-}
-
 template <typename T>
 __global__ __launch_bounds__(256) void sigmoid_attn_kernel(T* __restrict__ out, int64_t ld_out, float* __restrict__ part,
                                                            const float* __restrict__ q, const T* __restrict__ k_cache,
@@ -301,6 +274,156 @@ __global__ __launch_bounds__(256) void sigmoid_attn_kernel(T* __restrict__ out, 
     else
       part[((size_t)blockIdx.z * total_q + tok) * H * dv + (size_t)head * dv + c] = o[i];
   }
+}
+
+// The same on the matrix cores, for bf16 caches.  A workgroup = 64 query rows ((token, head) pairs of one request and ONE key/value
+// head: QT tokens x HB heads) in 4 waves of 16 rows, one key range.  Keys and values come through LDS in tiles of 64 rows, row-major,
+// 16-byte padded.  Per 16-key subtile and wave:
+//   S^T[16 keys x 16 rows] = K . Q^T     KC x v_mfma_f32_16x16x32_bf16   (Q fragments live in registers, rounded to bf16 once)
+//   weights in fp32 in the lane that holds the score (one query row, four keys): the B-operand layout of the second product;
+//   O^T[16 v x 16 rows] += V^T . P^T     VC x v_mfma_f32_16x16x16_bf16, V^T fragments read TRANSPOSED out of the row-major value
+//   tile (ds_read_b64_tr_b16).  There is no running maximum and nothing to rescale: weights are independent of each other.
+constexpr int kSKT = 64;
+
+__device__ __forceinline__ float capped_sigmoid(float s, float cap, float inv_cap, float bias) {
+  if (cap > 0.f) s = cap * (1.0f - 2.0f / (1.0f + __expf(2.0f * s * inv_cap)));  // cap * tanh(s / cap)
+  return 1.0f / (1.0f + __expf(-(s + bias)));
+}
+
+template <int KC, int VC>
+__global__ __launch_bounds__(256) void sigmoid_attn_mfma_kernel(bf16_t* __restrict__ out, int64_t ld_out, float* __restrict__ part,
+                                                                const float* __restrict__ q, const bf16_t* __restrict__ k_cache,
+                                                                const bf16_t* __restrict__ v_cache, const int* __restrict__ table,
+                                                                int64_t table_stride, const int* __restrict__ req_rows,
+                                                                const int* __restrict__ seq_lens, const int* __restrict__ cu_q, int B,
+                                                                int total_q, int H, int G, int d, int dv, float scale, float cap,
+                                                                const float* __restrict__ pb, float out_scale, int QT, int HB, int splits,
+                                                                int kvec, int vvec) {
+  constexpr int KS = KC * 32 + 8, VS = VC * 16 + 8;
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  uint16_t* sk = smem;               // [kSKT][KS]
+  uint16_t* sv = smem + kSKT * KS;   // [kSKT][VS]
+  __shared__ int s_req, s_tok0, s_cnt[256];
+  __shared__ int s_slot[2][kSKT];
+  find_group(cu_q, B, QT, s_cnt, &s_req, &s_tok0);
+  const int b = s_req;
+  if (b < 0) return;
+  const int rep = H / G, hblocks = (rep + HB - 1) / HB;
+  const int kvh = blockIdx.y / hblocks, h0 = kvh * rep + (blockIdx.y % hblocks) * HB, z = blockIdx.z;
+  const int q_len = cu_q[b + 1] - cu_q[b];
+  const int start = seq_lens[b] - q_len;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int r = wave * 16 + lr;
+  const int tl = s_tok0 + r / HB, hh = h0 + r % HB;
+  const bool valid = r < QT * HB && tl < q_len && hh < (kvh + 1) * rep;
+  const int tok = cu_q[b] + (valid ? tl : s_tok0);
+  const int head = valid ? hh : h0;
+  const int limit = valid ? start + tl : -1;
+  const int last_tok = min(s_tok0 + QT, q_len) - 1;
+  const int n_keys = start + last_tok + 1;
+  const int per = ((n_keys + splits - 1) / splits + kSKT - 1) / kSKT * kSKT;
+  const int k_begin = z * per, k_end = min(n_keys, k_begin + per);
+  const bool wave_live = __builtin_amdgcn_ballot_w64(valid) != 0;
+  bf16x8_t qf[KC];
+  {
+    const float* qrow = q + ((size_t)tok * H + head) * d;
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) {
+      const int k = kc * 32 + lg * 8;
+      Q4 v = (valid && k < d) ? load8(qrow + k, d - k, (d & 3) == 0) : Q4{0u, 0u, 0u, 0u};
+      qf[kc] = __builtin_bit_cast(bf16x8_t, v);
+    }
+  }
+  f32x4_t o[VC];
+#pragma unroll
+  for (int vt = 0; vt < VC; ++vt) o[vt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const float bias_h = pb ? pb[head] : 0.f, inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
+  const int* trow = table + (size_t)req_rows[b] * table_stride;
+  const size_t nkd = (size_t)G * d, nvd = (size_t)G * dv, ko = (size_t)kvh * d, vo = (size_t)kvh * dv;
+  // the next tile's rows are requested before the current tile's products: their latency hides under the MFMAs
+  constexpr int NK = (kSKT * KC * 4 + 255) / 256, NV = (kSKT * VC * 2 + 255) / 256;
+  Q4 pre_k[NK], pre_v[NV];
+  auto request = [&](int j0, int buf) {
+#pragma unroll
+    for (int u = 0; u < NK; ++u) {
+      const int e = u * 256 + threadIdx.x;
+      const int key = e / (KC * 4), k = (e - key * (KC * 4)) * 8;
+      pre_k[u] = Q4{0u, 0u, 0u, 0u};
+      if (e < kSKT * KC * 4 && j0 + key < k_end && k < d) pre_k[u] = load8(k_cache + (size_t)s_slot[buf][key] * nkd + ko + k, d - k, kvec != 0);
+    }
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int e = u * 256 + threadIdx.x;
+      const int key = e / (VC * 2), c = (e - key * (VC * 2)) * 8;
+      pre_v[u] = Q4{0u, 0u, 0u, 0u};
+      if (e < kSKT * VC * 2 && j0 + key < k_end && c < dv) pre_v[u] = load8(v_cache + (size_t)s_slot[buf][key] * nvd + vo + c, dv - c, vvec != 0);
+    }
+  };
+  if (threadIdx.x < kSKT && k_begin + (int)threadIdx.x < k_end) s_slot[0][threadIdx.x] = trow[k_begin + threadIdx.x];
+  __syncthreads();
+  if (k_begin < k_end) request(k_begin, 0);
+  int buf = 0;
+  for (int j0 = k_begin; j0 < k_end; j0 += kSKT, buf ^= 1) {
+    __syncthreads();
+    if (threadIdx.x < kSKT && j0 + kSKT + (int)threadIdx.x < k_end) s_slot[buf ^ 1][threadIdx.x] = trow[j0 + kSKT + threadIdx.x];
+#pragma unroll
+    for (int u = 0; u < NK; ++u) {
+      const int e = u * 256 + threadIdx.x;
+      const int key = e / (KC * 4), ch = e - key * (KC * 4);
+      if (e < kSKT * KC * 4) *reinterpret_cast<Q4*>(&sk[key * KS + ch * 8]) = pre_k[u];
+    }
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int e = u * 256 + threadIdx.x;
+      const int key = e / (VC * 2), ch = e - key * (VC * 2);
+      if (e < kSKT * VC * 2) *reinterpret_cast<Q4*>(&sv[key * VS + ch * 8]) = pre_v[u];
+    }
+    __syncthreads();
+    if (j0 + kSKT < k_end) request(j0 + kSKT, buf ^ 1);
+    if (!wave_live) continue;
+    constexpr int NKS = kSKT / 16;
+    s16x4_t pf[NKS];
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      f32x4_t sacc{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kc = 0; kc < KC; ++kc) {
+        const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(&sk[(ks * 16 + lr) * KS + kc * 32 + lg * 8]);
+        sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kc], sacc, 0, 0, 0);
+      }
+      float pe[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int j = j0 + ks * 16 + 4 * lg + c;
+        pe[c] = (j <= limit && j < k_end) ? capped_sigmoid(sacc[c] * scale, cap, inv_cap, bias_h) : 0.f;
+      }
+      const uint32_t p01 = bf16_bits(pe[0]) | (bf16_bits(pe[1]) << 16), p23 = bf16_bits(pe[2]) | (bf16_bits(pe[3]) << 16);
+      pf[ks] = __builtin_bit_cast(s16x4_t, uint2{p01, p23});
+    }
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      if (j0 + ks * 16 >= k_end) break;
+      const uint16_t* vbase = &sv[(ks * 16 + 4 * lg + (lr >> 2)) * VS + 4 * (lr & 3)];
+#pragma unroll
+      for (int vt = 0; vt < VC; ++vt) {
+        const s16x4_t vf = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(vbase + vt * 16));
+        o[vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pf[ks], o[vt], 0, 0, 0);
+      }
+    }
+  }
+  if (!valid) return;
+#pragma unroll
+  for (int vt = 0; vt < VC; ++vt)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int v = vt * 16 + 4 * lg + c;
+      if (v >= dv) continue;
+      if (splits == 1)
+        st(out + (size_t)tok * ld_out + (size_t)head * dv + v, o[vt][c] * out_scale);
+      else
+        part[((size_t)z * total_q + tok) * H * dv + (size_t)head * dv + v] = o[vt][c];
+    }
 }
 
 template <typename T>
@@ -457,15 +580,31 @@ __global__ __launch_bounds__(256) void gate_group_norm_kernel(T* __restrict__ ou
 }
 
 // ------------------------------------------------------------------------------------------------ activation
+// A thread takes 8 consecutive elements of a row (16-byte loads when `vec`), so the two softplus of the layer's numbers are paid once
+// per 8 elements.
 template <typename T>
 __global__ __launch_bounds__(256) void xielu_kernel(T* __restrict__ out, const T* __restrict__ z, int64_t ldz, const float* __restrict__ pq,
-                                                    int64_t total, int N) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= total) return;
-  const int64_t r = i / N;
+                                                    int64_t groups, int N, int vec) {
+  const int64_t gi = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (gi >= groups) return;
+  const int per_row = (N + 7) >> 3;
+  const int64_t r = gi / per_row;
+  const int c0 = (int)(gi - r * per_row) << 3, n = N - c0 < 8 ? N - c0 : 8;
   const float a = softplusf_(pq[0]), bneg = 0.5f + softplusf_(pq[1]);
-  const float x = ld(z + r * ldz + (i - r * N));
-  st(out + i, x > 0.f ? fmaf(a * x, x, 0.5f * x) : fmaf(bneg, expm1f(x) - x, 0.5f * x));
+  const T* src = z + r * ldz + c0;
+  T* dst = out + r * N + c0;
+  float x[8];
+  if (vec && n == 8) {
+    read8(src, x);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = i < n ? ld(src + i) : 0.f;
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float v = x[i] > 0.f ? fmaf(a * x[i], x[i], 0.5f * x[i]) : fmaf(bneg, expm1f(x[i]) - x[i], 0.5f * x[i]);
+    if (i < n) st(dst + i, v);
+  }
 }
 
 }  // namespace
@@ -552,6 +691,38 @@ int msgl_mix_sigmoid_attn(void* out, int64_t ld_out, const float* q, const void*
   MIX_REQUIRE(splits >= 1 && splits <= 1024 && (splits == 1 || workspace), "sigmoid_attn: %d splits need a workspace", splits);
   if (total_q == 0) return MSGL_MIX_OK;
   const int rep = H / G;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MSGL_MIX_BF16 && d <= 256 && dv <= 256) {
+    // matrix-core kernel: the smallest (KC, VC) instance that holds d <= 32 KC and dv <= 16 VC
+    int HBm = 1;
+    while (HBm * 2 <= rep && HBm * 2 <= 64) HBm *= 2;
+    const int QTm = 64 / HBm, hbl = (rep + HBm - 1) / HBm;
+    const int groups_m = (total_q + QTm - 1) / QTm + batch;
+    MIX_REQUIRE((int64_t)G * hbl <= 65535, "sigmoid_attn: too many heads");
+    const dim3 grid(groups_m, G * hbl, splits);
+    const int kvec = (((uintptr_t)k_cache & 15u) == 0 && d % 8 == 0) ? 1 : 0, vvec = (((uintptr_t)v_cache & 15u) == 0 && dv % 8 == 0) ? 1 : 0;
+#define SIG_CASE(KC, VC)                                                                                                                  \
+  if (d <= KC * 32 && dv <= VC * 16) {                                                                                                    \
+    const size_t lds_m = (size_t)kSKT * ((KC * 32 + 8) + (VC * 16 + 8)) * sizeof(uint16_t);                                               \
+    MIX_REQUIRE(ensure_lds((const void*)sigmoid_attn_mfma_kernel<KC, VC>, lds_m) == 0, "sigmoid_attn: LDS request refused");              \
+    hipLaunchKernelGGL((sigmoid_attn_mfma_kernel<KC, VC>), grid, dim3(256), lds_m, s, mp<bf16_t>(out), ld_out, workspace, q,              \
+                       cp<bf16_t>(k_cache), cp<bf16_t>(v_cache), table, table_stride, req_rows, seq_lens, cu_q, batch, total_q, H, G, d,  \
+                       dv, scale, softcap, pb, out_scale, QTm, HBm, splits, kvec, vvec);                                                  \
+    MIX_LAUNCHED("sigmoid_attn (matrix cores)");                                                                                          \
+    if (splits > 1) {                                                                                                                     \
+      hipLaunchKernelGGL(sigmoid_merge_kernel<bf16_t>, dim3(total_q), dim3(256), 0, s, mp<bf16_t>(out), ld_out, workspace, total_q,       \
+                         H * dv, splits, out_scale);                                                                                      \
+      MIX_LAUNCHED("sigmoid_attn merge");                                                                                                 \
+    }                                                                                                                                     \
+    return MSGL_MIX_OK;                                                                                                                   \
+  }
+    SIG_CASE(2, 4)
+    SIG_CASE(3, 6)
+    SIG_CASE(4, 8)
+    SIG_CASE(6, 12)
+    SIG_CASE(8, 16)
+#undef SIG_CASE
+  }
   int HB = 1;
   while (HB * 2 <= rep && HB * 2 <= kSigRows) HB *= 2;
   const int QT = kSigRows / HB, hblocks = (rep + HB - 1) / HB;
@@ -562,7 +733,6 @@ int msgl_mix_sigmoid_attn(void* out, int64_t ld_out, const float* q, const void*
   MIX_REQUIRE(lds <= 160 * 1024, "sigmoid_attn: heads of %d / %d do not fit LDS", d, dv);
   const int groups = (total_q + QT - 1) / QT + batch;  // every request may end with one partial group
   MIX_REQUIRE((int64_t)G * hblocks <= 65535, "sigmoid_attn: too many heads");
-  hipStream_t s = static_cast<hipStream_t>(stream);
   DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)sigmoid_attn_kernel<T>, lds) == 0, "sigmoid_attn: LDS request refused");
              hipLaunchKernelGGL(sigmoid_attn_kernel<T>, dim3(groups, G * hblocks, splits), dim3(256), lds, s, mp<T>(out), ld_out, workspace, q,
                                 cp<T>(k_cache), cp<T>(v_cache), table, table_stride, req_rows, seq_lens, cu_q, batch, total_q, H, G, d, dv,
@@ -626,10 +796,12 @@ int msgl_mix_gate_group_norm(void* out, int64_t ld_out, const float* y, const vo
 int msgl_mix_xielu(void* out, const void* z, int64_t ldz, const float* pq, int rows, int N, int dtype, void* stream) {
   MIX_REQUIRE(out && z && pq && rows >= 0 && N >= 1 && ldz >= N && dtype_ok(dtype), "xielu: bad arguments");
   if (rows == 0) return MSGL_MIX_OK;
-  const int64_t total = (int64_t)rows * N;
+  const int64_t groups = (int64_t)rows * ((N + 7) / 8);
+  const int es = dtype == MSGL_MIX_BF16 ? 2 : 4;
+  const int vec = (N % 8 == 0 && ldz % 8 == 0 && ((uintptr_t)z & 15u) == 0 && (es == 2 || ((uintptr_t)z & 31u) == 0)) ? 1 : 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  DISPATCH_T(dtype, hipLaunchKernelGGL(xielu_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, mp<T>(out), cp<T>(z), ldz, pq,
-                                       total, N);)
+  DISPATCH_T(dtype, hipLaunchKernelGGL(xielu_kernel<T>, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s, mp<T>(out), cp<T>(z), ldz, pq,
+                                       groups, N, vec);)
   MIX_LAUNCHED("xielu");
   return MSGL_MIX_OK;
 }

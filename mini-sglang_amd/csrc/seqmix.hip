@@ -107,37 +107,6 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const T* __restrict__ 
 }
 
 // ------------------------------------------------------------------------------------------------ latent attention
-// Which request and which of its QT-token groups workgroup `blockIdx.x` owns: group counts ceil(new tokens / QT) of up to 256
-// requests at a time, scanned by the whole workgroup (one pass of independent loads instead of one thread walking the batch).
-// Leaves request -1 for workgroups past the last group.  cnt: 256 ints of LDS; every thread of the (256-thread) workgroup calls.
-__device__ __forceinline__ void find_group(const int* __restrict__ cu_q, int B, int QT, int* cnt, int* s_req, int* s_tok0) {
-  const int tid = threadIdx.x;
-  if (tid == 0) *s_req = -1;
-  int base = 0;
-  for (int c0 = 0; c0 < B; c0 += 256) {
-    const int b = c0 + tid;
-    const int g = b < B ? (cu_q[b + 1] - cu_q[b] + QT - 1) / QT : 0;
-    cnt[tid] = g;
-    __syncthreads();
-    for (int off = 1; off < 256; off <<= 1) {
-      const int v = tid >= off ? cnt[tid - off] : 0;
-      __syncthreads();
-      cnt[tid] += v;
-      __syncthreads();
-    }
-    const int incl = cnt[tid], total = cnt[255];
-    const int target = (int)blockIdx.x - base;
-    if (b < B && target >= incl - g && target < incl) {
-      *s_req = b;
-      *s_tok0 = (target - (incl - g)) * QT;
-    }
-    __syncthreads();
-    if (target < total) break;
-    base += total;
-  }
-  __syncthreads();
-}
-
 // A sink is one more term exp(sink[h]) in a head's softmax denominator, with no key and no value.  With running maximum m
 // over the keys and M = max(m, sink): out = f o / (f l + w), f = exp(m - M), w = exp(sink - M)  (no sink: f = 1, w = 0).
 __device__ __forceinline__ float sink_factor(const float* __restrict__ sink, int head, float m) {
@@ -762,39 +731,7 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(TC* __restrict__ C, const 
 // current step's MFMAs.  LDS rows are 72 elements apart (144 B): the 16 lanes of a fragment read land on 16 different bank quads.  A wave
 // whose rows lie past the end of a (short) expert segment skips its MFMAs, so a decode step pays for the weight stream only.
 // An output element's k order is fixed, wherever its row sits in a segment: results do not depend on the batch around it.
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-struct __attribute__((aligned(16))) Q4 {
-  uint32_t x, y, z, w;
-};
 constexpr int kMT = 128, kMK = 64, kMLd = 72;
-
-__device__ __forceinline__ uint32_t bf16_bits(float v) {
-  bf16_t t;
-  st(&t, v);
-  return t.bits;
-}
-
-// eight consecutive k of one row as packed bf16; `n` of them exist (the rest read as zero); vec: 16-byte loads are legal
-__device__ __forceinline__ Q4 load8(const bf16_t* p, int n, bool vec) {
-  if (vec && n >= 8) return *reinterpret_cast<const Q4*>(p);
-  uint32_t e[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) e[i] = i < n ? p[i].bits : 0u;
-  return Q4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
-}
-__device__ __forceinline__ Q4 load8(const float* p, int n, bool vec) {
-  float f[8];
-  if (vec && n >= 8) {
-    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
-    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
-  } else {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = i < n ? p[i] : 0.f;
-  }
-  return Q4{bf16_bits(f[0]) | (bf16_bits(f[1]) << 16), bf16_bits(f[2]) | (bf16_bits(f[3]) << 16),
-            bf16_bits(f[4]) | (bf16_bits(f[5]) << 16), bf16_bits(f[6]) | (bf16_bits(f[7]) << 16)};
-}
 
 template <typename TA, typename TC>
 __global__ __launch_bounds__(256) void gemm_nt_mfma_kernel(TC* __restrict__ C, const TA* __restrict__ A, const bf16_t* __restrict__ Bm, int M,
@@ -907,8 +844,6 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma_kernel(TC* __restrict__ C, c
 // Softmax in fp32 per row, one step per 64-key tile: tile max across the four lane groups, running (m, l), O rescaled when
 // a row's max moved.
 // splits > 1 (decode: few rows, many keys): (m, l, O) partials per split, merged by latent_attn_merge_kernel.
-typedef __attribute__((ext_vector_type(4))) short s16x4_t;
-typedef __attribute__((address_space(3))) s16x4_t lds_s16x4_t;
 constexpr int kAKT = 64;
 
 template <int KC, int VC>

@@ -756,7 +756,7 @@ class HybridDecoder:
                            interleaved=a.interleaved, unit=True)
         mixops.sigmoid_attn(cat[:, : H * dv], q, kc, vc, ctx.page_table, md.req_rows, md.seq_lens, md.cu_seqlens_q, md.batch, H, G, d, dv,
                             a.scale, a.softcap, L.pb, out_scale=s.left_scale,
-                            splits=mixops.sigmoid_attn_splits(md.batch, T, md.max_seqlen_k))
+                            splits=mixops.sigmoid_attn_splits(md.batch, T, H, G, md.max_seqlen_k) if md.max_seqlen_q <= 16 else 1)
         # right: proj[:, n_left:] = z | x B C | dt
         z, xbc_raw, dt_raw = proj[:, n_left: n_left + inner], proj[:, n_left + inner: n_left + inner + C], proj[:, n_left + inner + C:]
         xbc = mixops.short_conv(xbc_raw, C, L.taps, kv.conv_state(i), md.cu_seqlens_q, md.seq_lens, md.req_rows, md.batch,

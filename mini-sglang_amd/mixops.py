@@ -532,12 +532,15 @@ def qk_prep(proj: torch.Tensor, bias: Optional[torch.Tensor], k_cache: torch.Ten
     return q
 
 
-def sigmoid_attn_splits(batch: int, total_q: int, max_keys: int) -> int:
-    """Key ranges per request for a step with few query tokens: enough workgroups to fill the chip, at least 256 keys each.  A
-    function of static sizes only, so a captured graph keeps its grid."""
-    if total_q >= 8 * batch and total_q >= 256:
-        return 1
-    return max(1, min(512 // max(total_q + batch, 1), max_keys // 256, 32))
+def sigmoid_attn_splits(batch: int, total_q: int, H: int, G: int, max_keys: int) -> int:
+    """Key ranges per request for a step with few query rows: enough workgroups to fill the chip, at least 256 keys each.  A
+    function of static sizes only (batch, rows, the LONGEST possible key count), so a captured graph keeps its grid."""
+    rep = H // G
+    hb = 1
+    while hb * 2 <= min(rep, 64):
+        hb *= 2
+    blocks = (-(-total_q // (64 // hb)) + batch) * G * -(-rep // hb)
+    return max(1, min(1024 // max(blocks, 1), max_keys // 256, 64))
 
 
 def sigmoid_attn(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, table: torch.Tensor, req_rows: torch.Tensor,

@@ -110,7 +110,7 @@ def kernel_rooflines(name: str, prompt: int, batch: int, device) -> dict:
         kc, vc = rnd(slots, G * D), rnd(slots, G * D)
         pb = torch.full((H,), -2.0, dtype=torch.float32, device=device)
         o = torch.empty(T, H * D, dtype=bf, device=device)
-        sp = mixops.sigmoid_attn_splits(reqs, T, ctx)
+        sp = mixops.sigmoid_attn_splits(reqs, T, H, G, ctx) if q_len <= 16 else 1
         us = _time_us(lambda: mixops.sigmoid_attn(o, q, kc, vc, table, rows, seq, cu, reqs, H, G, D, D, D ** -0.5, 50.0, pb, splits=sp))
         attn_bytes = reqs * ctx * 2 * G * D * 2 + T * H * D * (4 + 2)
         out[f"{phase}.sigmoid_attn"] = _entry(us, 4.0 * pairs * H * D, attn_bytes, MFMA_TFLOPS)
@@ -149,7 +149,7 @@ def kernel_rooflines(name: str, prompt: int, batch: int, device) -> dict:
         rate, dtb, skip = -torch.rand(Hs, device=device), torch.zeros(Hs, device=device), torch.ones(Hs, device=device)
         y = torch.empty(T, inner, dtype=torch.float32, device=device)
         chunks = chunk_list(q_len, reqs, 128)
-        us = _time_us(lambda: mixops.ssd(y, xbc, pr[:, inner + C + inner:], state, rate, dtb, skip, cu, seq, rows, reqs, Gs, chunks=chunks))
+        us = _time_us(lambda: mixops.ssd(y, xbc, pr[:, inner + C:], state, rate, dtb, skip, cu, seq, rows, reqs, Gs, chunks=chunks))
         out[f"{phase}.ssd"] = _entry(us, 5.0 * T * Hs * N * P, 2 * reqs * Hs * N * P * 4 + T * C * 4 + T * inner * 4, VALU_TFLOPS)
         lq = rnd(T, 4 * H * D, scale=0.5)
         lstate = torch.zeros(reqs, H, D, D, dtype=torch.float32, device=device)
