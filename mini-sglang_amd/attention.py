@@ -225,7 +225,7 @@ class MixAttnBackend:
 
     RECURRENT_CHUNK = 128
     DELTA_CHUNK = 256
-    SSD_CHUNK = 128
+    SSD_CHUNK = 64
 
     def __init__(self, config: Any, ctx: Any = None, *, tp_size: int = 1) -> None:
         ctx = ctx if ctx is not None else _core.get_global_ctx()

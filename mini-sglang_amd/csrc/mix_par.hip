@@ -16,8 +16,8 @@
 //                           both products on the matrix cores, weights in fp32; key ranges are plain partial sums
 //                           (sigmoid_merge_kernel adds them)
 //   sigmoid_attn_kernel     the same in plain fp32 (fp32 caches, heads past the matrix-core instances)
-//   ssd_kernel              S <- exp(rate dt) S + dt B x^T,  y = S^T C + D x per (request, head); a thread owns one column of S;
-//                           long portions as parallel chunks joined by ssd_scan_kernel
+//   ssd_kernel              S <- exp(rate dt) S + dt B x^T,  y = S^T C + D x per (request, head); four waves share the rows of a
+//                           state column; long portions as parallel chunks joined by ssd_scan_kernel
 //   gate_group_norm_kernel  (y * silu(z)) normed in equal groups of the row, times w
 //   xielu_kernel            z > 0: a z^2 + z / 2;  z <= 0: b (exp(z) - 1 - z) + z / 2
 #include "mix_common.h"
@@ -438,25 +438,26 @@ __global__ __launch_bounds__(256) void sigmoid_merge_kernel(T* __restrict__ out,
 }
 
 // ------------------------------------------------------------------------------------------------ state-space recurrence
-// Workgroup = (block of 64 value columns, head, request or chunk); a thread owns column e of the head's state S [N, P] (DP >= N
-// registers, the tail zero).  Per token:  dt = softplus(dt_raw + dt_bias[h]);  a = exp(rate[h] dt);  S <- a S + (dt x_e) B;
-// y_e = S . C + D[h] x_e.  Rows xbc = [x: H x P | B: G x N | C: G x N] (fp32); B and C of a token are the same for every lane and
-// are read through uniform addresses.
+// Workgroup = (block of 64 value columns, head, request or chunk), 4 waves; lane = column e of the head's state S [N, P], wave w
+// owns rows w R .. w R + R - 1 of that column in registers (4 R >= N, the tail zero).  Per token:
+//   dt = softplus(dt_raw + dt_bias[h]);  a = exp(rate[h] dt);  S <- a S + (dt x_e) B;  y_e = S . C + D[h] x_e
+// (the four waves' partial dot products are added in wave order).  Rows xbc = [x: H x P | B: G x N | C: G x N] (fp32); the B and C
+// entries a wave needs are the same for all its lanes and are read through uniform addresses.  16 tokens are staged at a time.
 // MODE 0  a request's whole portion from its state row (zero when the portion starts at position 0), state row written back.
 // Long portions are cut into chunks that run in parallel; over a chunk S_end = A S_start + L with A = exp(rate * sum of dt).
 // MODE 1  a chunk's L from zero and its sum of dt -> scratch[item], chunk_dt[item, h]; no outputs; the last chunk of a request is
 //         skipped (nothing follows it).  ssd_scan_kernel then walks a request's chunks: start[c + 1] = A_c start[c] + L_c.
 // MODE 2  a chunk's outputs from its start state (scratch[item] after the scan); the last chunk writes the state row.
-template <typename T, int DP, int MODE>
-__global__ __launch_bounds__(64) void ssd_kernel(float* __restrict__ out, const float* __restrict__ xbc, int64_t ld_x, const T* __restrict__ dt_raw,
-                                                 int64_t ld_dt, float* __restrict__ state, const float* __restrict__ rate,
-                                                 const float* __restrict__ dt_bias, const float* __restrict__ Dv, const int* __restrict__ cu_q,
-                                                 const int* __restrict__ seq_lens, const int* __restrict__ slots, int H, int G, int N, int P,
-                                                 const int* __restrict__ items, const int* __restrict__ item_first, float* __restrict__ scratch,
-                                                 float* __restrict__ chunk_dt) {
+template <typename T, int R, int MODE>
+__global__ __launch_bounds__(256) void ssd_kernel(float* __restrict__ out, const float* __restrict__ xbc, int64_t ld_x, const T* __restrict__ dt_raw,
+                                                  int64_t ld_dt, float* __restrict__ state, const float* __restrict__ rate,
+                                                  const float* __restrict__ dt_bias, const float* __restrict__ Dv, const int* __restrict__ cu_q,
+                                                  const int* __restrict__ seq_lens, const int* __restrict__ slots, int H, int G, int N, int P,
+                                                  const int* __restrict__ items, const int* __restrict__ item_first, float* __restrict__ scratch,
+                                                  float* __restrict__ chunk_dt) {
   constexpr int kStage = 16;
-  __shared__ float sx[kStage][64], sdt[kStage], sa[kStage];
-  const int h = blockIdx.y, lane = threadIdx.x, e = blockIdx.x * 64 + lane;
+  __shared__ float sx[kStage][64], sdt[kStage], sa[kStage], part[kStage][4][64];
+  const int h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, e = blockIdx.x * 64 + lane;
   int b, first, n_new;
   bool last_chunk = true;
   if (MODE == 0) {
@@ -472,66 +473,73 @@ __global__ __launch_bounds__(64) void ssd_kernel(float* __restrict__ out, const 
     if (MODE == 1 && last_chunk) return;
   }
   if (n_new <= 0) return;
-  const int grp = h / (H / G);
+  const int grp = h / (H / G), row0 = wave * R;
   const bool live = e < P;
-  float S[DP];
+  float S[R];
   if (MODE == 1) {
 #pragma unroll
-    for (int i = 0; i < DP; ++i) S[i] = 0.f;
+    for (int i = 0; i < R; ++i) S[i] = 0.f;
   } else {
     const bool fresh = MODE == 0 && seq_lens[b] == n_new;
     const float* Srow = MODE == 0 ? state + ((size_t)slots[b] * H + h) * N * P : scratch + ((size_t)blockIdx.z * H + h) * N * P;
 #pragma unroll
-    for (int i = 0; i < DP; ++i) S[i] = (!fresh && live && i < N) ? Srow[(size_t)i * P + e] : 0.f;
+    for (int i = 0; i < R; ++i) S[i] = (!fresh && live && row0 + i < N) ? Srow[(size_t)(row0 + i) * P + e] : 0.f;
   }
   const float r = rate[h], dskip = Dv[h], db = dt_bias[h];
   const size_t no = (size_t)H * P;
+  const bool full = row0 + R <= N;  // uniform over the wave
   float dt_sum = 0.f;
   for (int t0 = 0; t0 < n_new; t0 += kStage) {
     const int nt = n_new - t0 < kStage ? n_new - t0 : kStage;
     __syncthreads();
-    if (lane < nt) {
-      const float dt = softplusf_(ld(dt_raw + (size_t)(first + t0 + lane) * ld_dt + h) + db);
-      sdt[lane] = dt;
-      sa[lane] = expf(r * dt);
+    if (threadIdx.x < nt) {
+      const float dt = softplusf_(ld(dt_raw + (size_t)(first + t0 + threadIdx.x) * ld_dt + h) + db);
+      sdt[threadIdx.x] = dt;
+      sa[threadIdx.x] = expf(r * dt);
     }
-    for (int tt = 0; tt < nt; ++tt) sx[tt][lane] = live ? xbc[(size_t)(first + t0 + tt) * ld_x + (size_t)h * P + e] : 0.f;
+    for (int tt = wave; tt < nt; tt += 4) sx[tt][lane] = live ? xbc[(size_t)(first + t0 + tt) * ld_x + (size_t)h * P + e] : 0.f;
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
-      const float* __restrict__ Bp = xbc + (size_t)(first + t0 + tt) * ld_x + (size_t)H * P + (size_t)grp * N;
+      const float* __restrict__ Bp = xbc + (size_t)(first + t0 + tt) * ld_x + (size_t)H * P + (size_t)grp * N + row0;
       const float* __restrict__ Cp = Bp + (size_t)G * N;
-      const float a = sa[tt], xv = sx[tt][lane], u = sdt[tt] * xv;
+      const float a = sa[tt], u = sdt[tt] * sx[tt][lane];
       if (MODE == 1) dt_sum += sdt[tt];
       float y = 0.f;
-      if (N == DP) {
+      if (full) {
 #pragma unroll
-        for (int i = 0; i < DP; ++i) {
+        for (int i = 0; i < R; ++i) {
           S[i] = fmaf(a, S[i], u * Bp[i]);
           if (MODE != 1) y = fmaf(S[i], Cp[i], y);
         }
       } else {
 #pragma unroll
-        for (int i = 0; i < DP; ++i) {
-          if (i < N) {
+        for (int i = 0; i < R; ++i) {
+          if (row0 + i < N) {
             S[i] = fmaf(a, S[i], u * Bp[i]);
             if (MODE != 1) y = fmaf(S[i], Cp[i], y);
           }
         }
       }
-      if (MODE != 1 && live) out[(size_t)(first + t0 + tt) * no + (size_t)h * P + e] = fmaf(dskip, xv, y);
+      if (MODE != 1) part[tt][wave][lane] = y;
+    }
+    if (MODE == 1) continue;
+    __syncthreads();
+    for (int tt = wave; tt < nt; tt += 4) {
+      const float y = ((part[tt][0][lane] + part[tt][1][lane]) + part[tt][2][lane]) + part[tt][3][lane];
+      if (live) out[(size_t)(first + t0 + tt) * no + (size_t)h * P + e] = fmaf(dskip, sx[tt][lane], y);
     }
   }
   if (MODE == 1) {
     float* L = scratch + ((size_t)blockIdx.z * H + h) * N * P;
 #pragma unroll
-    for (int i = 0; i < DP; ++i)
-      if (live && i < N) L[(size_t)i * P + e] = S[i];
-    if (blockIdx.x == 0 && lane == 0) chunk_dt[(size_t)blockIdx.z * H + h] = dt_sum;
+    for (int i = 0; i < R; ++i)
+      if (live && row0 + i < N) L[(size_t)(row0 + i) * P + e] = S[i];
+    if (blockIdx.x == 0 && threadIdx.x == 0) chunk_dt[(size_t)blockIdx.z * H + h] = dt_sum;
   } else if (last_chunk) {
     float* Srow = state + ((size_t)slots[b] * H + h) * N * P;
 #pragma unroll
-    for (int i = 0; i < DP; ++i)
-      if (live && i < N) Srow[(size_t)i * P + e] = S[i];
+    for (int i = 0; i < R; ++i)
+      if (live && row0 + i < N) Srow[(size_t)(row0 + i) * P + e] = S[i];
   }
 }
 
@@ -757,14 +765,14 @@ int msgl_mix_ssd(float* out, const float* xbc, int64_t ld_x, const void* dt_raw,
 #define SSD_GO(DP)                                                                                                                        \
   if (N <= DP) {                                                                                                                          \
     DISPATCH_T(dtype, if (n_items == 0) {                                                                                                 \
-      hipLaunchKernelGGL((ssd_kernel<T, DP, 0>), dim3(cb, H, batch), dim3(64), 0, s, out, xbc, ld_x, cp<T>(dt_raw), ld_dt, state, rate,   \
+      hipLaunchKernelGGL((ssd_kernel<T, DP / 4, 0>), dim3(cb, H, batch), dim3(256), 0, s, out, xbc, ld_x, cp<T>(dt_raw), ld_dt, state, rate,   \
                          dt_bias, D, cu_q, seq_lens, slots, H, G, N, P, items, item_first, scratch, chunk_dt);                            \
     } else {                                                                                                                              \
-      hipLaunchKernelGGL((ssd_kernel<T, DP, 1>), dim3(cb, H, n_items), dim3(64), 0, s, out, xbc, ld_x, cp<T>(dt_raw), ld_dt, state, rate, \
+      hipLaunchKernelGGL((ssd_kernel<T, DP / 4, 1>), dim3(cb, H, n_items), dim3(256), 0, s, out, xbc, ld_x, cp<T>(dt_raw), ld_dt, state, rate, \
                          dt_bias, D, cu_q, seq_lens, slots, H, G, N, P, items, item_first, scratch, chunk_dt);                            \
       hipLaunchKernelGGL(ssd_scan_kernel, dim3(H, batch, (N * P + 255) / 256), dim3(256), 0, s, state, scratch, chunk_dt, rate, cu_q,     \
                          seq_lens, slots, item_first, H, N * P);                                                                          \
-      hipLaunchKernelGGL((ssd_kernel<T, DP, 2>), dim3(cb, H, n_items), dim3(64), 0, s, out, xbc, ld_x, cp<T>(dt_raw), ld_dt, state, rate, \
+      hipLaunchKernelGGL((ssd_kernel<T, DP / 4, 2>), dim3(cb, H, n_items), dim3(256), 0, s, out, xbc, ld_x, cp<T>(dt_raw), ld_dt, state, rate, \
                          dt_bias, D, cu_q, seq_lens, slots, H, G, N, P, items, item_first, scratch, chunk_dt);                            \
     })                                                                                                                                    \
     MIX_LAUNCHED("ssd");                                                                                                                  \

@@ -74,12 +74,14 @@ def _entry(us: float, flops: float, byts: float, flop_peak: float) -> dict:
             "of_roofline": round(max(flops / us / 1e6 / flop_peak, byts / us / 1e6 / HBM_TBS), 4)}
 
 
-def kernel_rooflines(name: str, prompt: int, batch: int, device) -> dict:
+def kernel_rooflines(name: str, prompt: int, batch: int, device, ssd_chunk: int = 0) -> dict:
     """Each new kernel alone at the size's shapes, beside its like kernel of the other hybrid decoders: microseconds and the share
     of the roofline that bounds it (matrix cores for a prompt portion's attention products, the fp32 vector rate for the
     recurrences, HBM for everything a decode step streams)."""
     from mini_sglang_amd import mixops
+    from mini_sglang_amd.attention import MixAttnBackend
 
+    ssd_chunk = ssd_chunk or MixAttnBackend.SSD_CHUNK
     W, order, H, G, D, R, r, Hs, P, N, Gs, taps, ff, V, _, _, _ = SIZES[name]
     bf = torch.bfloat16
     out = {}
@@ -148,14 +150,14 @@ def kernel_rooflines(name: str, prompt: int, batch: int, device) -> dict:
         state = torch.zeros(reqs, Hs, N, P, dtype=torch.float32, device=device)
         rate, dtb, skip = -torch.rand(Hs, device=device), torch.zeros(Hs, device=device), torch.ones(Hs, device=device)
         y = torch.empty(T, inner, dtype=torch.float32, device=device)
-        chunks = chunk_list(q_len, reqs, 128)
+        chunks = chunk_list(q_len, reqs, ssd_chunk)
         us = _time_us(lambda: mixops.ssd(y, xbc, pr[:, inner + C:], state, rate, dtb, skip, cu, seq, rows, reqs, Gs, chunks=chunks))
         out[f"{phase}.ssd"] = _entry(us, 5.0 * T * Hs * N * P, 2 * reqs * Hs * N * P * 4 + T * C * 4 + T * inner * 4, VALU_TFLOPS)
         lq = rnd(T, 4 * H * D, scale=0.5)
         lstate = torch.zeros(reqs, H, D, D, dtype=torch.float32, device=device)
         decay = torch.full((H,), 0.97, dtype=torch.float32, device=device)
         od = torch.empty(T, H * D, dtype=torch.float32, device=device)
-        us = _time_us(lambda: mixops.lightning(od, lq, lstate, decay, cu, seq, rows, reqs, chunks=chunks))
+        us = _time_us(lambda: mixops.lightning(od, lq, lstate, decay, cu, seq, rows, reqs, chunks=chunk_list(q_len, reqs, 128)))
         out[f"{phase}.lightning (like)"] = _entry(us, 4.0 * T * H * D * D, 2 * reqs * H * D * D * 4 + T * 3 * H * D * 2 + T * H * D * 4, VALU_TFLOPS)
         cat = torch.empty(T, H * D + inner, dtype=bf, device=device)
         nw = torch.ones(inner, dtype=torch.float32, device=device)
@@ -198,6 +200,7 @@ def main(argv=None) -> None:
     ap.add_argument("--no-twin", action="store_true", help="skip the post-norm hybrid decoder of equal size")
     ap.add_argument("--no-kernels", action="store_true")
     ap.add_argument("--no-engine", action="store_true", help="kernel rooflines only")
+    ap.add_argument("--ssd-chunk", type=int, default=0, help="piece size of long portions in the state-space kernel's own measurement")
     args = ap.parse_args(argv)
     from mini_sglang_amd.hybrid import HybridConfig, givavik_config
 
@@ -217,7 +220,7 @@ def main(argv=None) -> None:
                                                        device)
                 print(f"[givavik bench] {name} twin: " + json.dumps(entry["post_norm_hybrid"]), flush=True)
         if not args.no_kernels:
-            entry["kernels"] = kernel_rooflines(name, args.prompt, args.batch, device)
+            entry["kernels"] = kernel_rooflines(name, args.prompt, args.batch, device, args.ssd_chunk)
         report["sizes"][name] = entry
     print(json.dumps(report))
 
