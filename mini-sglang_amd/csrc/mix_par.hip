@@ -2,7 +2,7 @@
 // by side; mixers: latent attention with a sink, or sigmoid attention beside a state-space layer), gfx950, wave = 64 lanes.
 // Third translation unit of libmsgl_mix.so; C ABI in include/msgl_mix.h.
 //
-// Precision contract (as in seqmix.hip): the residual stream, every norm, rotary angles, attention scores and weights, step
+// Precision rules (as in seqmix.hip): the residual stream, every norm, rotary angles, attention scores and weights, step
 // sizes, decays and the recurrent state are fp32 in registers and in memory; tensors that feed a matrix product are stored in
 // the model dtype T (bf16 or fp32).  With T = float every kernel here is true 32-bit.
 //

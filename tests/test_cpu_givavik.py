@@ -1,4 +1,4 @@
-"""CPU-side checks of the parallel-residual hybrid decoder (Givavik): configuration reader, registry, checkpoint round trip,
+"""CPU-side tests of the parallel-residual hybrid decoder (Givavik): configuration reader, registry, checkpoint round trip,
 cache layout, and the plain restatement's own consistency (tests/givavik_oracle.py)."""
 from __future__ import annotations
 

@@ -32,11 +32,11 @@ def givavik_json(name: str) -> dict:
     layers, last_l = [], None
     for i, c in enumerate(order):
         if c == "P":
-            left = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "softcap": 50.0, "rot": {"base": 5e5, "dims": D // 2}}
+            left = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "softcap": 30.0, "rot": {"base": 1e6, "dims": D // 2}}
             right = {"heads": Hs, "vdim": P, "state": N, "groups": Gs, "conv": taps, "norm_groups": Gs}
             layers.append({"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}, "mlp": mlp})
         else:
-            m = {"heads": H, "dim": D, "rot_dim": r, "vdim": D, "kv_rank": R, "scale": (D + r) ** -0.5, "rot": {"base": 5e5, "dims": r}}
+            m = {"heads": H, "dim": D, "rot_dim": r, "vdim": D, "kv_rank": R, "scale": (D + r) ** -0.5, "rot": {"base": 1e6, "dims": r}}
             if c == "B":
                 m["kv_from"] = last_l
             else:
@@ -113,7 +113,7 @@ def kernel_rooflines(name: str, prompt: int, batch: int, device, ssd_chunk: int 
         pb = torch.full((H,), -2.0, dtype=torch.float32, device=device)
         o = torch.empty(T, H * D, dtype=bf, device=device)
         sp = mixops.sigmoid_attn_splits(reqs, T, H, G, ctx) if q_len <= 16 else 1
-        us = _time_us(lambda: mixops.sigmoid_attn(o, q, kc, vc, table, rows, seq, cu, reqs, H, G, D, D, D ** -0.5, 50.0, pb, splits=sp))
+        us = _time_us(lambda: mixops.sigmoid_attn(o, q, kc, vc, table, rows, seq, cu, reqs, H, G, D, D, D ** -0.5, 30.0, pb, splits=sp))
         attn_bytes = reqs * ctx * 2 * G * D * 2 + T * H * D * (4 + 2)
         out[f"{phase}.sigmoid_attn"] = _entry(us, 4.0 * pairs * H * D, attn_bytes, MFMA_TFLOPS)
         src = rnd(T, H * D + H, scale=0.3)
@@ -135,7 +135,7 @@ def kernel_rooflines(name: str, prompt: int, batch: int, device, ssd_chunk: int 
         proj = rnd(T, n_left, scale=0.5)
         bias = torch.zeros(n_left, dtype=torch.float32, device=device)
         from mini_sglang_amd.hybrid import plain_rotary_table
-        cs = plain_rotary_table(D // 2, 5e5, ctx, device)
+        cs = plain_rotary_table(D // 2, 1e6, ctx, device)
         out_loc = table.view(-1)[: T] if reqs == 1 else table[:, ctx - 1].contiguous()
         us = _time_us(lambda: mixops.qk_prep(proj, bias, kc, vc, out_loc, pos, cs, 1e-5, H, G, D, D, interleaved=True, unit=True))
         out[f"{phase}.qk_prep"] = _entry(us, 0.0, T * (n_left * 2 + H * D * 4 + 2 * G * D * 2), VALU_TFLOPS)
