@@ -70,49 +70,127 @@ __global__ __launch_bounds__(256) void embed_scaled_kernel(float* __restrict__ x
 // so it equals what that token's own workgroup computes), state[req_rows[b]] for a portion's first token, zero at position 0.
 // The last token of every request leaves its h in staging[b]; commit_rows_kernel moves it to the state row after the forward
 // (a portion's first and last token run in different workgroups of this launch, so the state row cannot be replaced here).
-template <typename T>
+// A workgroup takes TT consecutive tokens; only the first of them has to rebuild the row before it.
+__device__ __forceinline__ void write8(float* p, const float (&f)[8]) {
+  *reinterpret_cast<float4*>(p) = float4{f[0], f[1], f[2], f[3]};
+  *reinterpret_cast<float4*>(p + 4) = float4{f[4], f[5], f[6], f[7]};
+}
+__device__ __forceinline__ void write8(bf16_t* p, const float (&f)[8]) {
+  bf16_t t[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) st(&t[i], f[i]);
+  *reinterpret_cast<uint4*>(p) = uint4{(uint32_t)t[0].bits | ((uint32_t)t[1].bits << 16), (uint32_t)t[2].bits | ((uint32_t)t[3].bits << 16),
+                                       (uint32_t)t[4].bits | ((uint32_t)t[5].bits << 16), (uint32_t)t[6].bits | ((uint32_t)t[7].bits << 16)};
+}
+
+// VEC: W is a multiple of 8 and every row is 16-byte aligned -- a thread takes 8 consecutive columns at a time with 16-byte loads
+// and stores; otherwise one column at a time.  Either way a thread only ever touches its own columns of the LDS rows.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void shift_norm_kernel(const float* __restrict__ x_in, float* __restrict__ x_out, const T* __restrict__ y0,
                                                          int64_t ld0, const float* __restrict__ v0, const T* __restrict__ y1, int64_t ld1,
                                                          const float* __restrict__ v1, const float* __restrict__ bias,
                                                          const float* __restrict__ w, float w_off, const float* __restrict__ shift, T* __restrict__ h_out,
                                                          T* __restrict__ g_out, const float* __restrict__ state, float* __restrict__ staging,
                                                          const int* __restrict__ positions, const int* __restrict__ cu_q,
-                                                         const int* __restrict__ req_rows, int batch, float eps, int W) {
-  extern __shared__ float srow[];  // W (this token's row) + W (the previous token's)
+                                                         const int* __restrict__ req_rows, int batch, float eps, int W, int rows, int TT) {
+  extern __shared__ __attribute__((aligned(16))) float srow[];  // two rows of W: this token's and the one before it
   __shared__ float red[4];
-  float* cur = srow;
-  float* prv = srow + W;
-  const int t = blockIdx.x;
+  constexpr int kStep = VEC ? 8 : 1;
+  auto vec_of = [](const float* __restrict__ p, int c, float (&f)[kStep]) {  // kStep columns of a per-column fp32 vector
+    if constexpr (VEC) {
+      read8(p + c, f);
+    } else {
+      f[0] = p[c];
+    }
+  };
   auto row_of = [&](int tt, float* dst, bool store) {
     float ss = 0.f;
-    for (int i = threadIdx.x; i < W; i += 256) {
-      float s = x_in[(size_t)tt * W + i];
-      if (bias) s += bias[i];
-      if (y0) s = fmaf(v0 ? v0[i] : 1.f, ld(y0 + (size_t)tt * ld0 + i), s);
-      if (y1) s = fmaf(v1 ? v1[i] : 1.f, ld(y1 + (size_t)tt * ld1 + i), s);
-      if (store) x_out[(size_t)tt * W + i] = s;
-      dst[i] = s;
-      ss += s * s;
+    for (int c = threadIdx.x * kStep; c < W; c += 256 * kStep) {
+      float s[kStep], a[kStep], m[kStep];
+      if constexpr (VEC) {
+        read8(x_in + (size_t)tt * W + c, s);
+      } else {
+        s[0] = x_in[(size_t)tt * W + c];
+      }
+      if (bias) {
+        vec_of(bias, c, a);
+#pragma unroll
+        for (int u = 0; u < kStep; ++u) s[u] += a[u];
+      }
+      if (y0) {
+        if constexpr (VEC) read8(y0 + (size_t)tt * ld0 + c, a); else a[0] = ld(y0 + (size_t)tt * ld0 + c);
+#pragma unroll
+        for (int u = 0; u < kStep; ++u) m[u] = 1.f;
+        if (v0) vec_of(v0, c, m);
+#pragma unroll
+        for (int u = 0; u < kStep; ++u) s[u] = fmaf(m[u], a[u], s[u]);
+      }
+      if (y1) {
+        if constexpr (VEC) read8(y1 + (size_t)tt * ld1 + c, a); else a[0] = ld(y1 + (size_t)tt * ld1 + c);
+#pragma unroll
+        for (int u = 0; u < kStep; ++u) m[u] = 1.f;
+        if (v1) vec_of(v1, c, m);
+#pragma unroll
+        for (int u = 0; u < kStep; ++u) s[u] = fmaf(m[u], a[u], s[u]);
+      }
+      if (store) {
+        if constexpr (VEC) write8(x_out + (size_t)tt * W + c, s); else x_out[(size_t)tt * W + c] = s[0];
+      }
+#pragma unroll
+      for (int u = 0; u < kStep; ++u) {
+        dst[c + u] = s[u];
+        ss += s[u] * s[u];
+      }
     }
     return 1.0f / sqrtf(block_sum256(ss, red) / (float)W + eps);
   };
-  const float inv = row_of(t, cur, x_out != nullptr);
-  if (!shift) {
-    for (int i = threadIdx.x; i < W; i += 256) st(h_out + (size_t)t * W + i, cur[i] * inv * (w[i] + w_off));
-    return;
-  }
-  const int b = request_of(cu_q, batch, t);
-  const bool last = t == cu_q[b + 1] - 1;
-  const int mode = positions[t] == 0 ? 0 : (t > cu_q[b] ? 1 : 2);  // uniform over the workgroup
-  float inv_p = 0.f;
-  if (mode == 1) inv_p = row_of(t - 1, prv, false);
-  const float* srow_state = state + (size_t)req_rows[b] * W;
-  for (int i = threadIdx.x; i < W; i += 256) {
-    const float wi = w[i] + w_off, h = cur[i] * inv * wi;
-    const float hp = mode == 0 ? 0.f : (mode == 1 ? prv[i] * inv_p * wi : srow_state[i]);
-    if (h_out) st(h_out + (size_t)t * W + i, h);
-    st(g_out + (size_t)t * W + i, h + (hp - h) * shift[i]);
-    if (last) staging[(size_t)b * W + i] = h;
+  // a workgroup walks TT consecutive tokens: from the second on, the row before is still in LDS and is not read again
+  float inv_before = 0.f;
+  for (int k = 0; k < TT; ++k) {
+    const int t = blockIdx.x * TT + k;
+    if (t >= rows) break;
+    float* cur = srow + (k & 1) * W;
+    float* prv = srow + ((k & 1) ^ 1) * W;
+    const float inv = row_of(t, cur, x_out != nullptr);
+    if (!shift) {
+      for (int c = threadIdx.x * kStep; c < W; c += 256 * kStep) {
+        float h[kStep], wv[kStep];
+        vec_of(w, c, wv);
+#pragma unroll
+        for (int u = 0; u < kStep; ++u) h[u] = cur[c + u] * inv * (wv[u] + w_off);
+        if constexpr (VEC) write8(h_out + (size_t)t * W + c, h); else st(h_out + (size_t)t * W + c, h[0]);
+      }
+      continue;
+    }
+    const int b = request_of(cu_q, batch, t);
+    const bool last = t == cu_q[b + 1] - 1;
+    const int mode = positions[t] == 0 ? 0 : (t > cu_q[b] ? 1 : 2);  // uniform over the workgroup
+    float inv_p = inv_before;
+    if (mode == 1 && k == 0) inv_p = row_of(t - 1, prv, false);
+    const float* srow_state = state + (size_t)req_rows[b] * W;
+    for (int c = threadIdx.x * kStep; c < W; c += 256 * kStep) {
+      float h[kStep], g[kStep], wv[kStep], sv[kStep], pv[kStep];
+      vec_of(w, c, wv);
+      vec_of(shift, c, sv);
+      if (mode == 2) vec_of(srow_state, c, pv);
+#pragma unroll
+      for (int u = 0; u < kStep; ++u) {
+        const float wi = wv[u] + w_off;
+        h[u] = cur[c + u] * inv * wi;
+        const float hp = mode == 0 ? 0.f : (mode == 1 ? prv[c + u] * inv_p * wi : pv[u]);
+        g[u] = h[u] + (hp - h[u]) * sv[u];
+      }
+      if constexpr (VEC) {
+        if (h_out) write8(h_out + (size_t)t * W + c, h);
+        write8(g_out + (size_t)t * W + c, g);
+        if (last) write8(staging + (size_t)b * W + c, h);
+      } else {
+        if (h_out) st(h_out + (size_t)t * W + c, h[0]);
+        st(g_out + (size_t)t * W + c, g[0]);
+        if (last) staging[(size_t)b * W + c] = h[0];
+      }
+    }
+    inv_before = inv;
   }
 }
 
@@ -648,10 +726,26 @@ int msgl_mix_shift_norm(const float* x_in, float* x_out, const void* y0, int64_t
   }
   if (rows == 0) return MSGL_MIX_OK;
   const size_t lds = (size_t)2 * W * sizeof(float);
+  // long batches: a workgroup takes 2 consecutive tokens and re-reads one row in two instead of every row (measured: 4 and 8
+  // tokens per workgroup gain nothing more, the serial walk costs what the saved reads give); short ones keep a workgroup per
+  // token (the arithmetic of a token is the same either way)
+  const int TT = (shift && rows >= 1024) ? 2 : 1;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)shift_norm_kernel<T>, lds) == 0, "shift_norm: two rows of %d do not fit LDS", W);
-             hipLaunchKernelGGL(shift_norm_kernel<T>, dim3(rows), dim3(256), lds, s, x_in, x_out, cp<T>(y0), ld0, v0, cp<T>(y1), ld1, v1, bias,
-                                w, w_off, shift, mp<T>(h_out), mp<T>(g_out), state, staging, positions, cu_q, req_rows, batch, eps, W);)
+  auto al16 = [](const void* p) { return ((uintptr_t)p & 15u) == 0; };
+  const int es = dtype == MSGL_MIX_BF16 ? 2 : 4;
+  const bool vec = W % 8 == 0 && al16(w) && al16(shift) && al16(bias) && al16(v0) && al16(v1) && al16(state) && al16(x_in) && al16(x_out) && al16(h_out) && al16(g_out) && al16(staging) && al16(y0) && al16(y1) &&
+                   (!y0 || (ld0 * es) % 16 == 0) && (!y1 || (ld1 * es) % 16 == 0);
+#define SN_LAUNCH(VEC)                                                                                                                          \
+  DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)shift_norm_kernel<T, VEC>, lds) == 0, "shift_norm: two rows of %d do not fit LDS", W); \
+             hipLaunchKernelGGL((shift_norm_kernel<T, VEC>), dim3((rows + TT - 1) / TT), dim3(256), lds, s, x_in, x_out, cp<T>(y0), ld0, v0,    \
+                                cp<T>(y1), ld1, v1, bias, w, w_off, shift, mp<T>(h_out), mp<T>(g_out), state, staging, positions, cu_q,         \
+                                req_rows, batch, eps, W, rows, TT);)
+  if (vec) {
+    SN_LAUNCH(true)
+  } else {
+    SN_LAUNCH(false)
+  }
+#undef SN_LAUNCH
   MIX_LAUNCHED("shift_norm");
   return MSGL_MIX_OK;
 }

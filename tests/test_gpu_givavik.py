@@ -346,6 +346,16 @@ def test_long_portions_run_as_parallel_chunks_fp32():
     assert rel(got["a"], whole) < 2e-5
 
 
+def test_very_long_portion_against_shorter_ones_fp32():
+    """A 2300-token portion (the norm-and-shift launch then walks two tokens per workgroup and keeps the row before in LDS)
+    beside a short request, against the same tokens in portions that take the one-token-per-workgroup path."""
+    eng, _ = engine_for(FULL, torch.float32, max_tokens=4096)
+    a, b = tokens_of(2300, FULL["vocab"], 32), tokens_of(7, FULL["vocab"], 33)
+    long = replay(eng, [[("b", b[:3], False), ("a", a, True)], [("b", b[3:], True)]])
+    short = replay(eng, [[("a", a[:700], False)], [("a", a[700:1600], False), ("b", b, True)], [("a", a[1600:], True)]])
+    assert rel(long["a"], short["a"]) < 2e-5 and rel(long["b"], short["b"]) < 2e-5
+
+
 def test_long_decoding_fp32():
     """A short prompt, then 260 tokens one by one: keys far back stay visible, the states carry everything else."""
     cfg = config([pair(mlp=dense()), lat(mlp=None), pair(s_heads=2, s_vdim=20, state=12, norm_groups=2), lat(kv_from=1, mlp=dense())])
