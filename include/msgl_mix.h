@@ -27,7 +27,7 @@ extern "C" {
 #define MSGL_MIX_ACT_NONE 0
 #define MSGL_MIX_ACT_RELU2 1 /* max(z, 0)^2 */
 
-#define MSGL_MIX_ABI_VERSION 3
+#define MSGL_MIX_ABI_VERSION 4
 
 const char* msgl_mix_last_error(void);
 int msgl_mix_abi_version(void);
@@ -141,12 +141,12 @@ int msgl_mix_window_attn(void* out, const void* src, int64_t ld_src, int g_off, 
                          void* stream);
 
 /* Causal convolution over time per channel, then SiLU: out[t, c] = silu(bias[c] + sum_j taps[c, j] in[pos - (n - 1) + j, c]) (fp32;
- * bias in T, may be null);
+ * out_t: the same rows in T; either may be null; bias in T, may be null);
  * inputs of this forward are src[t, 0 : C], earlier ones come from state[slots[b]] ([n - 1, C] in T per request: the inputs
  * of the n - 1 positions before the portion), positions before 0 count as zero.  The first `unit_heads` groups of d channels
  * leave as unit vectors (x / sqrt(sum x^2 + 1e-6)), the first `scaled_heads` of them times d^-1/2.  A second launch moves every
  * request's state on to its last n - 1 inputs. */
-int msgl_mix_short_conv(float* out, const void* src, int64_t ld_src, const void* taps, const void* bias, void* state, const int* cu_q,
+int msgl_mix_short_conv(float* out, void* out_t, const void* src, int64_t ld_src, const void* taps, const void* bias, void* state, const int* cu_q,
                         const int* seq_lens, const int* slots, int batch, int total, int C, int n, int unit_heads, int scaled_heads, int d,
                         int dtype, void* stream);
 
@@ -192,7 +192,8 @@ int msgl_mix_commit_rows(float* dst, int64_t dst_stride, const float* src, int64
                          int* prev_tok, const int* ids, const int* cu_q, void* stream);
 
 /* Projection row [q: H x d | k: G x d | v: G x dv | ...] (+ bias: fp32, same layout, may be null): the first rot_dims entries of
- * every q and k head turn (cos_sin and pairing as in msgl_mix_latent_prep), with unit != 0 every q and k head is divided by its
+ * every q and k head turn (cos_sin and pairing as in msgl_mix_latent_prep), with bit 0 of `unit` every q and k head, with bit 1
+ * every v head is divided by its
  * root mean square; q -> q_out (fp32 [tokens, H * d]), k and v -> cache rows at out_loc ([slots, G * d], [slots, G * dv], T). */
 int msgl_mix_qk_prep(const void* proj, int64_t ld_proj, const float* bias, float* q_out, void* k_cache, void* v_cache, const int* out_loc,
                      const int* positions, const float* cos_sin, int rot_dims, int interleaved, int unit, float eps, int tokens, int H,
@@ -225,6 +226,51 @@ int msgl_mix_gate_group_norm(void* out, int64_t ld_out, const float* y, const vo
 /* out = z > 0 ? a z^2 + z / 2 : b (exp(z) - 1 - z) + z / 2 with a = softplus(pq[0]), b = 1/2 + softplus(pq[1]) (pq: 2 floats on the
  * device); z rows ldz apart, out rows of N. */
 int msgl_mix_xielu(void* out, const void* z, int64_t ldz, const float* pq, int rows, int N, int dtype, void* stream);
+
+/* ---- looped pre-norm hybrid decoders (csrc/mix_scan.hip) ---- */
+
+/* Closes a sublayer and opens the next.  row = x_in + mult * (sum of the p0 rows of y0[t] and the p1 rows of y1[t]) + add -> x_out
+ * (fp32, a buffer other than x_in; y0 [rows, p0, W], y1 [rows, p1, W] in T, add fp32 [W]; each may be absent);  h = row with every
+ * one of `groups` equal parts divided by its own root mean square (eps inside the root), times w (T [W]);  h_out[t] (T) = h[t] +
+ * sum_j taps[c, j] h[t - (n - 1) + j] (taps T [W, n], null: h itself).  With n > 1 the rows are the new tokens of `batch` requests
+ * (cu_q, seq_lens as in msgl_mix_latent_attn): rows before a portion come from state[slots[b]] (fp32 [n - 1, W] per request: the h
+ * of the n - 1 positions before the portion), rows before position 0 are zero, and every request's new state rows are left in
+ * staging[b] (fp32 [batch, n - 1, W]) for msgl_mix_commit_rows.  cu_q null: plain rows (n must be 1). */
+int msgl_mix_norm_conv(const float* x_in, float* x_out, const void* y0, int p0, const void* y1, int p1, float mult, const float* add,
+                       const void* w, int groups, float eps, const void* taps, int n, const float* state, float* staging, void* h_out,
+                       const int* cu_q, const int* seq_lens, const int* slots, int batch, int rows, int W, int dtype, void* stream);
+
+/* Selective scan per (request, channel c): dt = softplus(dt_in[t, c] + dt_bias[c]); S[c, n] <- exp(dt A[c, n]) S[c, n] + dt x[t, c]
+ * B[t, n]; y = sum_n S[c, n] C[t, n] + D[c] x[t, c]; out[t, c] = y silu(z[t, c]).  x, z, dt_in: T rows of C channels (row strides
+ * given); bc: T rows [B: N | C: N]; A = -exp(A_log) fp32 [C, N]; state: fp32 [slots, C, N], row slots[b], zero for a request whose
+ * first new token is at position 0; out: T [tokens, C].  n_items > 0: chunks as in msgl_mix_lightning (over a chunk S_end =
+ * exp(A sum dt) S_start + L); scratch: fp32, n_items * C * (N + 1) floats. */
+int msgl_mix_selective_scan(void* out, const void* x, int64_t ld_x, const void* z, int64_t ld_z, const void* dt_in, int64_t ld_dt,
+                            const void* bc, int64_t ld_bc, const float* A, const float* dt_bias, const float* D, float* state,
+                            const int* cu_q, const int* seq_lens, const int* slots, int batch, int C, int N, int dtype, int n_items,
+                            const int* items, const int* item_first, float* scratch, void* stream);
+
+/* Softmax attention over the last `window` keys (window <= 0: all earlier keys) with a sink: out[t, h] = sum_j p_j v_j, p_j =
+ * exp(s_j) / (sum over visible keys of exp(s) + exp(sink[h])), s_j = scale q_h . k_j; sink fp32 [H] or null.  Query head h reads
+ * key/value head h / (H / G).  q: fp32 [tokens, H * d]; caches and requests as in msgl_mix_sigmoid_attn; `splits` > 1 cuts the
+ * visible keys into ranges joined by a second launch (workspace: fp32, msgl_mix_sink_attn_workspace_floats). */
+int msgl_mix_sink_attn_workspace_floats(int total_q, int H, int dv, int splits);
+int msgl_mix_sink_attn(void* out, int64_t ld_out, const float* q, const void* k_cache, const void* v_cache, const int* table,
+                       int64_t table_stride, const int* req_rows, const int* seq_lens, const int* cu_q, int batch, int total_q, int H, int G,
+                       int d, int dv, float scale, int window, const float* sink, int dtype, int splits, float* workspace, void* stream);
+
+/* Router on fp32 logits z [tokens, E]: the `top` largest win (ties: lowest index), the weight of a choice is sigmoid(its logit)
+ * -> ids int32 [tokens, top], wts fp32 [tokens, top]. */
+int msgl_mix_route_sigmoid(int* ids, float* wts, const float* z, int tokens, int E, int top, void* stream);
+
+/* out[t * top + k, :] = wts[t, k] * h[t, :] (T rows of W): the inputs of experts that are weighted before they run. */
+int msgl_mix_scale_rows(void* out, const void* h, const float* wts, int tokens, int top, int W, int dtype, void* stream);
+
+/* out (T [rows, N]) = o (fp32 [rows, N]) * sigmoid(g) (T rows ld_g apart). */
+int msgl_mix_sigmoid_gate(void* out, const float* o, const void* g, int64_t ld_g, int rows, int N, int dtype, void* stream);
+
+/* x <- cap * tanh(x / cap) in place (T rows of N, ld apart). */
+int msgl_mix_softcap(void* x, int64_t ld, int rows, int N, float cap, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

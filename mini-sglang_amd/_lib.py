@@ -20,7 +20,7 @@ HIP_SO = LIB_DIR / "libmsgl_hip.so"
 COMM_SO = LIB_DIR / "libmsgl_comm.so"
 GEMM_SO = LIB_DIR / "libmsgl_gemm.so"
 MIX_SO = LIB_DIR / "libmsgl_mix.so"
-MIX_ABI_VERSION = 3
+MIX_ABI_VERSION = 4
 
 BF16, FP16, F32 = 0, 1, 2
 UNIQUE_ID_BYTES = 128
@@ -161,7 +161,7 @@ MIX_SIGNATURES = {
     "msgl_mix_kv_store": (_i, [_p, _p, _p, _p, _l, _i, _i, _i, _i, _p, _l, _p, _i, _i, _p]),
     "msgl_mix_window_attn_workspace_floats": (_i, [_i, _i, _i, _i]),
     "msgl_mix_window_attn": (_i, [_p, _p, _l, _i, _p, _p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p, _i, _i, _p, _p]),
-    "msgl_mix_short_conv": (_i, [_p, _p, _l, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "msgl_mix_short_conv": (_i, [_p, _p, _p, _l, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "msgl_mix_delta_rule": (_i, [_p, _p, _p, _p, _l, _p, _l, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
     "msgl_mix_head_gated_norm": (_i, [_p, _p, _p, _l, _p, _f, _i, _i, _i, _i, _i, _p]),
     "msgl_mix_embed_scaled": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _p, _f, _i, _i, _i, _i, _i, _i, _p]),
@@ -173,6 +173,14 @@ MIX_SIGNATURES = {
     "msgl_mix_ssd": (_i, [_p, _p, _l, _p, _l, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
     "msgl_mix_gate_group_norm": (_i, [_p, _l, _p, _p, _l, _p, _f, _i, _i, _i, _f, _i, _p]),
     "msgl_mix_xielu": (_i, [_p, _p, _l, _p, _i, _i, _i, _p]),
+    "msgl_mix_norm_conv": (_i, [_p, _p, _p, _i, _p, _i, _f, _p, _p, _i, _f, _p, _i, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _p]),
+    "msgl_mix_selective_scan": (_i, [_p, _p, _l, _p, _l, _p, _l, _p, _l, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
+    "msgl_mix_sink_attn_workspace_floats": (_i, [_i, _i, _i, _i]),
+    "msgl_mix_sink_attn": (_i, [_p, _l, _p, _p, _p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _p, _i, _i, _p, _p]),
+    "msgl_mix_route_sigmoid": (_i, [_p, _p, _p, _i, _i, _i, _p]),
+    "msgl_mix_scale_rows": (_i, [_p, _p, _p, _i, _i, _i, _i, _p]),
+    "msgl_mix_sigmoid_gate": (_i, [_p, _p, _p, _l, _i, _i, _i, _p]),
+    "msgl_mix_softcap": (_i, [_p, _l, _i, _i, _f, _i, _p]),
 }
 
 

@@ -226,6 +226,7 @@ class MixAttnBackend:
     RECURRENT_CHUNK = 128
     DELTA_CHUNK = 256
     SSD_CHUNK = 64
+    SCAN_CHUNK = 64
 
     def __init__(self, config: Any, ctx: Any = None, *, tp_size: int = 1) -> None:
         ctx = ctx if ctx is not None else _core.get_global_ctx()
@@ -253,6 +254,8 @@ class MixAttnBackend:
             lists.append(("delta_chunks", self.DELTA_CHUNK))
         if int(q.max()) >= 2 * self.SSD_CHUNK and "state_space" in self._kinds:
             lists.append(("ssd_chunks", self.SSD_CHUNK))
+        if int(q.max()) >= 2 * self.SCAN_CHUNK and "mamba1" in self._kinds:
+            lists.append(("scan_chunks", self.SCAN_CHUNK))
         pieces = [-(-q // c) for _, c in lists]
         extra = sum(3 * int(p.sum()) + bs + 1 for p in pieces)
         host = torch.empty(3 * bs + 1 + extra, dtype=torch.int32, pin_memory=True)

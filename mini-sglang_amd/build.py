@@ -46,7 +46,7 @@ HIP_SOURCES = [
     "gemm_ro.hip",
     "comm_p2p.hip",
 ]
-MIX_SOURCES = ["seqmix.hip", "mix_delta.hip", "mix_par.hip"]
+MIX_SOURCES = ["seqmix.hip", "mix_delta.hip", "mix_par.hip", "mix_scan.hip"]
 COMM_SOURCES = ["comm.cpp"]
 GEMM_SOURCES = ["gemm.cpp"]
 

@@ -512,7 +512,8 @@ __global__ __launch_bounds__(256) void window_merge_kernel(T* __restrict__ out, 
 // The first `unit_heads` groups of d channels are made unit vectors (x / sqrt(sum x^2 + 1e-6)); the first `scaled_heads` of them
 // are also multiplied by d^-1/2.
 template <typename T>
-__global__ __launch_bounds__(256) void short_conv_kernel(float* __restrict__ out, const T* __restrict__ src, int64_t ld_src,
+__global__ __launch_bounds__(256) void short_conv_kernel(float* __restrict__ out, T* __restrict__ out_t, const T* __restrict__ src,
+                                                         int64_t ld_src,
                                                          const T* __restrict__ taps, const T* __restrict__ bias,
                                                          const T* __restrict__ state, const int* __restrict__ cu_q,
                                                          const int* __restrict__ seq_lens, const int* __restrict__ slots, int batch, int C,
@@ -543,7 +544,10 @@ __global__ __launch_bounds__(256) void short_conv_kernel(float* __restrict__ out
     for (int i = lane; i < d; i += 64) row[h * d + i] *= f;
   }
   __syncthreads();
-  for (int c = tid; c < C; c += 256) out[(size_t)t * C + c] = row[c];
+  if (out)
+    for (int c = tid; c < C; c += 256) out[(size_t)t * C + c] = row[c];
+  if (out_t)
+    for (int c = tid; c < C; c += 256) st(out_t + (size_t)t * C + c, row[c]);
 }
 
 // After short_conv_kernel: the state of every request in the batch moves on to its last n - 1 inputs.  Thread = (request, channel).
@@ -935,10 +939,10 @@ int msgl_mix_window_attn(void* out, const void* src, int64_t ld_src, int g_off, 
   return MSGL_MIX_OK;
 }
 
-int msgl_mix_short_conv(float* out, const void* src, int64_t ld_src, const void* taps, const void* bias, void* state, const int* cu_q,
+int msgl_mix_short_conv(float* out, void* out_t, const void* src, int64_t ld_src, const void* taps, const void* bias, void* state, const int* cu_q,
                         const int* seq_lens, const int* slots, int batch, int total, int C, int n, int unit_heads, int scaled_heads, int d,
                         int dtype, void* stream) {
-  MIX_REQUIRE(out && src && taps && cu_q && seq_lens && slots && dtype_ok(dtype), "short_conv: null pointer / dtype");
+  MIX_REQUIRE((out || out_t) && src && taps && cu_q && seq_lens && slots && dtype_ok(dtype), "short_conv: null pointer / dtype");
   MIX_REQUIRE(batch >= 0 && total >= 0 && C >= 1 && n >= 1 && n <= 17 && ld_src >= C && (n == 1 || state),
               "short_conv: bad sizes C %d taps %d", C, n);
   MIX_REQUIRE(unit_heads >= 0 && scaled_heads >= 0 && scaled_heads <= unit_heads && d >= 1 && (int64_t)unit_heads * d <= C,
@@ -947,7 +951,7 @@ int msgl_mix_short_conv(float* out, const void* src, int64_t ld_src, const void*
   const size_t lds = (size_t)C * sizeof(float);
   hipStream_t s = static_cast<hipStream_t>(stream);
   DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)short_conv_kernel<T>, lds) == 0, "short_conv: row of %d does not fit LDS", C);
-             hipLaunchKernelGGL(short_conv_kernel<T>, dim3(total), dim3(256), lds, s, out, cp<T>(src), ld_src, cp<T>(taps), cp<T>(bias),
+             hipLaunchKernelGGL(short_conv_kernel<T>, dim3(total), dim3(256), lds, s, out, mp<T>(out_t), cp<T>(src), ld_src, cp<T>(taps), cp<T>(bias),
                                 cp<T>(state), cu_q, seq_lens, slots, batch, C, n, unit_heads, scaled_heads, d);
              if (n > 1) hipLaunchKernelGGL(conv_state_kernel<T>, dim3((C + 255) / 256, batch), dim3(256), 0, s, mp<T>(state), cp<T>(src),
                                            ld_src, cu_q, slots, C, n);)

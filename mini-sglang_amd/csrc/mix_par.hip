@@ -212,7 +212,8 @@ __global__ __launch_bounds__(256) void commit_rows_kernel(float* __restrict__ ds
 // ------------------------------------------------------------------------------------------------ q / k preparation of grouped attention
 // One workgroup per token.  proj row = [q: H x d | k: G x d | v: G x dv | ...] (+ bias, fp32, same layout, may be null).  The first
 // rd entries of every q and k head turn by the token's angles (cos_sin row = cos | sin halves of rd / 2; pairs (2i, 2i + 1) when
-// `interleaved`, else (i, i + rd / 2)); with unit != 0 every head is then divided by its root mean square (eps inside the root).
+// `interleaved`, else (i, i + rd / 2)); with bit 0 of `unit` every q and k head is then divided by its root mean square (eps inside
+// the root), with bit 1 every v head.
 // q -> q_out (fp32 [tokens, H * d]); k, v -> the cache rows at out_loc (T).
 template <typename T>
 __global__ __launch_bounds__(256) void qk_prep_kernel(const T* __restrict__ proj, int64_t ld_proj, const float* __restrict__ bias,
@@ -243,7 +244,7 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const T* __restrict__ proj
     row[e] = v;
   }
   __syncthreads();
-  if (unit) {
+  if (unit & 1) {
     for (int hh = wave; hh < H + G; hh += 4) {
       float ss = 0.f;
       for (int i = lane; i < d; i += 64) ss = fmaf(row[hh * d + i], row[hh * d + i], ss);
@@ -256,6 +257,19 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const T* __restrict__ proj
   for (int e = threadIdx.x; e < H * d; e += 256) q_out[(size_t)t * H * d + e] = row[e];
   for (int e = threadIdx.x; e < G * d; e += 256) st(k_cache + slot * G * d + e, row[H * d + e]);
   const size_t vo = (size_t)(H + G) * d;
+  if (unit & 2) {  // every value head divided by its root mean square
+    for (int g = wave; g < G; g += 4) {
+      float ss = 0.f;
+      for (int i = lane; i < dv; i += 64) {
+        const float v = ld(src + vo + (size_t)g * dv + i) + (bias ? bias[vo + (size_t)g * dv + i] : 0.f);
+        ss = fmaf(v, v, ss);
+      }
+      const float f = 1.0f / sqrtf(wave_sum(ss) / (float)dv + eps);
+      for (int i = lane; i < dv; i += 64)
+        st(v_cache + slot * G * dv + (size_t)g * dv + i, (ld(src + vo + (size_t)g * dv + i) + (bias ? bias[vo + (size_t)g * dv + i] : 0.f)) * f);
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < G * dv; e += 256) st(v_cache + slot * G * dv + e, ld(src + vo + e) + (bias ? bias[vo + e] : 0.f));
 }
 

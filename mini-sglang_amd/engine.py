@@ -147,9 +147,9 @@ def determine_num_pages(free_before: int, free_after: int, cfg: EngineConfig) ->
     if cfg.num_page_override is not None:
         return cfg.num_page_override
     if isinstance(m, HybridConfig):  # one shared latent row per token and caching layer; the recurrent states are a fixed cost
-        cache_per_page = max(HybridCache.bytes_per_page(m.layers, cfg.page_size, cfg.dtype), 1)
-        free_after -= HybridCache.state_bytes(m.layers, cfg.max_running_req + 1, cfg.dtype,
-                                              shift_width=m.hidden_size if m.token_shift else 0)
+        cache_per_page = max(HybridCache.bytes_per_page(m.cache_layers, cfg.page_size, cfg.dtype), 1)
+        free_after -= HybridCache.state_bytes(m.cache_layers, cfg.max_running_req + 1, cfg.dtype,
+                                              shift_width=m.hidden_size if m.token_shift else 0, conv_in=(m.conv_taps, m.hidden_size))
     else:
         cache_per_page = (2 * m.head_dim * heads_per_rank(m.num_kv_heads, cfg.tp_size, replicate=True) * cfg.page_size
                           * torch.empty((), dtype=cfg.dtype).element_size() * m.num_layers)

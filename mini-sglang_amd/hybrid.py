@@ -52,7 +52,29 @@ parallel           two mixers on the same g, their results scaled and added:
                    Both mixers share one input projection and one output projection (their outputs side by side in one row).
 feed-forward       W_down xielu(W_up h) with two learned numbers per layer.
 
-Kernels: csrc/seqmix.hip, csrc/mix_delta.hip and csrc/mix_par.hip through mixops.py; plain projections through the library GEMM
+A fourth scheme, `pre_norm_conv` (the Piladra design): plain pre-norm residuals with a multiplier, norms in groups, a short causal
+convolution in front of every sublayer, and a run of layers that is repeated with the same weights:
+
+stream             x_0 = embed[token];  per layer  x <- x + m mixer(c1(norm1(x))),  x <- x + m ff(c2(norm2(x)));  a norm divides every
+                   one of `groups` equal parts of a row by its own root mean square, then multiplies by w;  c(h)[t] = h[t] + sum_j
+                   taps[:, j] h[t - (n - 1) + j] per channel (zero before the sequence; the last n - 1 normed rows of every sublayer are
+                   part of a request's state).  Layers start .. stop - 1 run `times` times in a row with the same weights, every pass
+                   with cache and state of its own; before the first layer of pass t the vector step[t] is added to x.  Output:
+                   final norm, head matrix, logits <- cap tanh(logits / cap).
+latent attention   as above with the rotated parts split in halves, an unscaled rotation, and the concatenated heads multiplied by
+                   sigmoid(W_g h) before the output projection.
+sink_attention     H query heads over G key/value heads, rotation of the leading entries of each head (frequencies rescaled by
+                   wavelength: short ones kept, long ones divided by a factor, a linear blend between), every value head divided by
+                   its root mean square before it is cached, keys 0 <= i - j < window visible, softmax with one more term
+                   exp(sink_h) in the denominator.  Cached per token: k [G d] and the normed v [G dv].
+mamba1             in-projection [x | z], causal convolution (+ bias) + SiLU over x, W_x x = [dt | B | C], dt = softplus(W_dt dt +
+                   bias), S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n, y_c = sum_n S[c, n] C_n + D_c x_c, y silu(z), output
+                   projection.  State per request: S [inner, state] in fp32 and the last taps - 1 inputs of the convolution.
+feed-forward       W_down (silu(W_gate h) * (W_up h)), or routed experts of that form: scores = sigmoid(router logits), the `top`
+                   largest chosen, a chosen expert runs on score * h (the weight enters BEFORE the expert, so the choices' outputs are
+                   summed as they are), plus a shared expert that every token runs.
+
+Kernels: csrc/seqmix.hip, csrc/mix_delta.hip, csrc/mix_par.hip and csrc/mix_scan.hip through mixops.py; plain projections through the library GEMM
 (mixops.linear).
 """
 from __future__ import annotations
@@ -76,7 +98,9 @@ class MoeSpec:
     keep: int = 1
     gated: bool = False             # expert = W_down (silu(W_gate h) * (W_up h)) instead of W_down relu(W_up h)^2
     pick: str = "scores"            # "scores": softmax over all experts, corrected group-limited choice; "logits": the largest
-                                    # logits (+ bias) win and the weights are the softmax over the winners
+                                    # logits (+ bias) win and the weights are the softmax over the winners; "sigmoid_input": the
+                                    # largest logits win, weight = sigmoid(logit), and it multiplies the expert's INPUT
+    shared_ff: int = 0              # inner size of a shared expert that every token runs (0: none)
 
 
 @dataclass(frozen=True)
@@ -84,11 +108,13 @@ class DenseFfSpec:
     ff: int
     act: str = "poly_norm"          # "poly_norm": c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3 with N = divide a row by its root mean square;
                                     # "xielu": softplus(p) z^2 + z / 2 above zero, (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2 below
+                                    # "silu_gate": W_down (silu(W_gate h) * (W_up h))
 
 
 @dataclass(frozen=True)
 class LayerSpec:
-    kind: str                       # "latent_attention" | "lightning" | "attention" | "delta" | "channel_delta" | "parallel";
+    kind: str                       # "latent_attention" | "lightning" | "attention" | "delta" | "channel_delta" | "parallel" |
+                                    # "sink_attention" | "mamba1";
                                     # inside a "parallel" pair: "sigmoid_attention" | "state_space"
     heads: int
     dim: int                        # unrotated query/key size per head (lightning: query/key size)
@@ -116,11 +142,15 @@ class LayerSpec:
     right: Optional["LayerSpec"] = None
     left_scale: float = 1.0
     right_scale: float = 1.0
+    out_gate: bool = False          # latent attention: the concatenated heads are multiplied by sigmoid(W_g h)
+    v_norm: bool = False            # sink attention: every value head is divided by its root mean square before it is cached
+    dt_rank: int = 0                # mamba1: inner size of the two-step step-size projection
     # state space: heads x vdim = inner size, dim = state size per head, kv_heads = groups of B / C, conv = taps
+    # mamba1: heads = 1, vdim = inner size (channels), dim = state size per channel, conv = taps
 
     @property
     def recurrent(self) -> bool:
-        return self.kind in ("lightning", "delta", "channel_delta", "state_space") or \
+        return self.kind in ("lightning", "delta", "channel_delta", "state_space", "mamba1") or \
             (self.kind == "parallel" and (self.left.recurrent or self.right.recurrent))
 
 
@@ -140,10 +170,33 @@ class HybridConfig:
     embed_scale: float = 1.0        # parallel_shift: the embedding row is multiplied by this
     pair_embed: Optional[Tuple[int, int, int]] = None  # (buckets, multiplier of the previous id, multiplier of the id) of the pair table
     token_shift: bool = False       # every layer's mixer reads a blend of this token's and the previous token's normed row
+    # "pre_norm_conv": x + m f(conv(norm(x))), norms in groups, a looped run of layers, capped logits, own head
+    norm_groups: int = 1            # a norm divides each of this many equal parts of a row by its own root mean square
+    conv_taps: int = 0              # taps of the causal convolution in front of every sublayer (0: none)
+    residual_mult: float = 1.0
+    logit_softcap: float = 0.0      # logits <- cap tanh(logits / cap); 0 = none
+    loop: Optional[Tuple[int, int, int]] = None   # (start, stop, times): layers start .. stop - 1 run `times` times in a row
 
     @property
     def num_layers(self) -> int:
         return len(self.layers)
+
+    @property
+    def runs(self) -> Tuple[Tuple[int, Optional[int]], ...]:
+        """(layer, pass number if the layer opens a pass of the loop else None) in the order the layers run."""
+        n = len(self.layers)
+        if self.loop is None:
+            return tuple((i, None) for i in range(n))
+        a, b, times = self.loop
+        out: List[Tuple[int, Optional[int]]] = [(i, None) for i in range(a)]
+        for t in range(times):
+            out += [(i, t if i == a else None) for i in range(a, b)]
+        return tuple(out + [(i, None) for i in range(b, n)])
+
+    @property
+    def cache_layers(self) -> Tuple[LayerSpec, ...]:
+        """One spec per layer RUN: every pass of a looped layer has cache rows and state of its own."""
+        return tuple(self.layers[i] for i, _ in self.runs)
 
     @staticmethod
     def from_json(cfg: Dict[str, Any], name: str = "Nidorax") -> "HybridConfig":
@@ -277,6 +330,73 @@ def givavik_config(cfg: Dict[str, Any], name: str = "Givavik") -> HybridConfig:
                         name=name, residual="parallel_shift", embed_scale=float(e.get("scale", 1.0)), pair_embed=pair, token_shift=True)
 
 
+def piladra_config(cfg: Dict[str, Any], name: str = "Piladra") -> HybridConfig:
+    """config.json of a Piladra model -> HybridConfig."""
+    layers: List[LayerSpec] = []
+    for i, entry in enumerate(cfg["layers"]):
+        m, kind, mlp = entry["mixer"], entry["type"], entry.get("mlp")
+        ff = None
+        if mlp is not None:
+            if mlp.get("kind") == "dense":
+                ff = DenseFfSpec(ff=int(mlp["ff"]), act="silu_gate")
+            elif mlp.get("kind") == "moe":
+                r, sh = mlp["router"], mlp.get("shared")
+                ff = MoeSpec(experts=int(r["experts"]), top=int(r["top"]), ff=int(mlp["expert"]["ff"]), gated=True, pick="sigmoid_input",
+                             shared_ff=int(sh["ff"]) if sh else 0)
+                if not 1 <= ff.top <= ff.experts:
+                    raise ValueError(f"layer {i}: top {ff.top} of {ff.experts} experts")
+            else:
+                raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+        if kind == "latent_attention":
+            r = int(m["rot_dim"])
+            dims, base = _rot(m, r)
+            if dims != r or r % 2:
+                raise ValueError(f"layer {i}: the rotated part has {r} entries, the rotation turns {dims}")
+            layers.append(LayerSpec(kind="latent_attention", heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), rot_dim=r,
+                                    kv_rank=int(m["kv_rank"]), scale=float(m["scale"]), rot_dims=dims, rot_base=base, out_gate=True, mlp=ff))
+        elif kind == "attention":
+            H, G = int(m["heads"]), int(m.get("kv_heads", m["heads"]))
+            dims, base = _rot(m, 0)
+            sc = (m.get("rot") or {}).get("scaling")
+            if H % G or dims % 2 or dims > int(m["dim"]):
+                raise ValueError(f"layer {i}: head / rotation sizes do not divide")
+            layers.append(LayerSpec(kind="sink_attention", heads=H, kv_heads=G, dim=int(m["dim"]), vdim=int(m["vdim"]), scale=float(m["scale"]),
+                                    window=int((m.get("mask") or {}).get("size", 0)), rot_dims=dims, rot_base=base,
+                                    rot_scaling=None if not sc else tuple(sorted((k, float(v)) for k, v in sc.items())),
+                                    sink=True, v_norm=True, mlp=ff))
+        elif kind == "mamba1":
+            layers.append(LayerSpec(kind="mamba1", heads=1, dim=int(m["state"]), vdim=int(m["inner"]), conv=int(m["conv"]),
+                                    dt_rank=int(m["dt_rank"]), mlp=ff))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+    loop = cfg.get("loop")
+    lp = None
+    if loop:
+        lp = (int(loop["start"]), int(loop["stop"]), int(loop["times"]))
+        if not (0 <= lp[0] <= lp[1] <= len(layers) and lp[2] >= 1):
+            raise ValueError(f"loop {lp} over {len(layers)} layers")
+    W, groups = int(cfg["width"]), int(cfg["norm"].get("groups", 1))
+    if W % groups:
+        raise ValueError(f"a row of {W} in {groups} groups")
+    return HybridConfig(vocab_size=int(cfg["vocab"]), hidden_size=W, layers=tuple(layers), rms_norm_eps=float(cfg["norm"]["eps"]), name=name,
+                        residual="pre_norm_conv", norm_groups=groups, conv_taps=int((cfg.get("canon") or {}).get("taps", 0)),
+                        residual_mult=float(cfg.get("residual_mult", 1.0)), logit_softcap=float(cfg.get("logit_softcap") or 0.0), loop=lp)
+
+
+def wavelength_scaled_rotary_table(dims: int, base: float, scaling: Optional[Dict[str, float]], max_position: int, device) -> torch.Tensor:
+    """fp32 [max_position, dims] = cos | sin of position * f_i, f_i = base^(-2i / dims) rescaled by wavelength l = 2 pi / f: kept where
+    l < original / high, divided by `factor` where l > original / low, blended linearly in original / l between; float64, rounded once."""
+    f = float(base) ** (-2.0 * torch.arange(dims // 2, dtype=torch.float64) / dims)
+    if scaling:
+        factor, low, high, orig = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+        wave = 2.0 * math.pi / f
+        blend = (orig / wave - low) / (high - low) if high != low else torch.zeros_like(f)
+        mixed = (1.0 - blend) * f / factor + blend * f
+        f = torch.where(wave < orig / high, f, torch.where(wave > orig / low, f / factor, mixed))
+    ang = torch.arange(max_position, dtype=torch.float64)[:, None] * f[None, :]
+    return torch.cat((ang.cos(), ang.sin()), dim=-1).to(torch.float32).to(device)
+
+
 def plain_rotary_table(dims: int, base: float, max_position: int, device) -> torch.Tensor:
     """fp32 [max_position, dims] = cos | sin of position * base^(-2i / dims), i < dims / 2; angles in float64, rounded once."""
     f = float(base) ** (-2.0 * torch.arange(dims // 2, dtype=torch.float64) / dims)
@@ -297,7 +417,8 @@ def rotary_table(spec: LayerSpec, max_position: int, device) -> torch.Tensor:
 class _Layer:
     __slots__ = ("spec", "w_in", "o", "norm1", "norm2", "uk_t", "uv", "c_norm", "cos_sin", "out_norm", "decay", "router",
                  "bias", "up", "down", "talk", "lam", "taps", "rate", "dt_bias", "a2", "g2", "act", "depth_w",
-                 "sink", "ls1", "ls2", "shift", "in_bias", "out_bias", "pb", "skip", "conv_b", "sum_bias")
+                 "sink", "ls1", "ls2", "shift", "in_bias", "out_bias", "pb", "skip", "conv_b", "sum_bias", "canon1", "canon2", "w_x", "w_dt",
+                 "sh_up", "sh_down")
 
     def __init__(self, spec: LayerSpec) -> None:
         self.spec = spec
@@ -326,7 +447,8 @@ class HybridDecoder:
         W = cfg.hidden_size
         self.pre_norm = cfg.residual == "pre_norm_depth"
         self.parallel = cfg.residual == "parallel_shift"
-        self.embed_norm = self.head = self.pair_table = None
+        self.conv_stream = cfg.residual == "pre_norm_conv"
+        self.embed_norm = self.head = self.pair_table = self.loop_step = None
         self.embed = w(cfg.vocab_size, W, std=1.0)
         self.final_norm = w(W, std=0.1)
         self.layers: List[_Layer] = []
@@ -364,15 +486,36 @@ class HybridDecoder:
                 # one output projection over the row [attention heads | state-space channels]
                 L.o = w(W, H * dv + inner, std=(H * dv + inner) ** -0.5)
                 L.out_bias = f32(W, std=0.1)
+            elif spec.kind == "mamba1":
+                inner, N, dr = spec.vdim, spec.dim, spec.dt_rank
+                L.w_in = w(2 * inner, W, std=W ** -0.5)           # x | z
+                L.taps = w(inner, spec.conv, std=spec.conv ** -0.5)
+                L.conv_b = w(inner, std=0.1)
+                L.w_x = w(dr + 2 * N, inner, std=inner ** -0.5)   # dt | B | C
+                L.w_dt = w(inner, dr, std=dr ** -0.5)
+                L.dt_bias, L.skip = f32(inner, std=0.5, mean=-2.0), f32(inner, std=0.3, mean=1.0)
+                L.rate = -torch.exp(f32(inner, N, std=0.5))       # A = -exp(A_log)
+                L.o = w(W, inner, std=inner ** -0.5)
+            elif spec.kind == "sink_attention":
+                G = spec.kv_heads
+                L.w_in = w(H * d + G * d + G * dv, W, std=W ** -0.5)  # q | k | v
+                L.o = w(W, H * dv, std=(H * dv) ** -0.5)
+                L.sink = f32(H, std=1.0)
+                if spec.rot_dims:
+                    key = ("wave", spec.rot_dims, spec.rot_base, spec.rot_scaling)
+                    if key not in tables:
+                        tables[key] = wavelength_scaled_rotary_table(spec.rot_dims, spec.rot_base, dict(spec.rot_scaling) if spec.rot_scaling else None,
+                                                                     self.max_position, device)
+                    L.cos_sin = tables[key]
             elif spec.kind == "latent_attention":
                 r, R = spec.rot_dim, spec.kv_rank
-                L.w_in = w(H * (d + r) + (0 if spec.kv_from is not None else R + r), W, std=W ** -0.5)
+                L.w_in = w(H * (d + r) + (0 if spec.kv_from is not None else R + r) + (H * dv if spec.out_gate else 0), W, std=W ** -0.5)
                 L.uk_t = w(H, R, d, std=R ** -0.5)   # W_uk per head, transposed: q_abs = q_unrotated @ uk_t[h]^T
                 L.uv = w(H, dv, R, std=R ** -0.5)
                 L.o = w(W, H * dv, std=(H * dv) ** -0.5)
                 L.c_norm = None if spec.kv_from is not None else (1.0 + w(R, std=0.1).float()).to(dtype)
                 L.sink = f32(H, std=1.0) if spec.sink else None
-                if spec.interleaved:
+                if spec.interleaved or self.conv_stream:
                     L.cos_sin = plain_table(spec.rot_dims, spec.rot_base)
                 else:
                     key = (spec.rot_dims, spec.rot_base, spec.rot_scaling)
@@ -407,14 +550,22 @@ class HybridDecoder:
             if isinstance(m, MoeSpec):
                 L.norm2 = w(W, std=0.1)
                 L.router = w(m.experts, W, std=W ** -0.5)
-                L.bias = w(m.experts, std=0.01)
+                L.bias = None if m.pick == "sigmoid_input" else w(m.experts, std=0.01)
                 L.up = w(m.experts, (2 if m.gated else 1) * m.ff, W, std=W ** -0.5)  # gated: every expert's gate rows, then its up rows
                 L.down = w(m.experts, W, m.ff, std=m.ff ** -0.5)
             elif isinstance(m, DenseFfSpec):
                 L.norm2 = None if self.parallel else w(W, std=0.1)
-                L.up = w(m.ff, W, std=W ** -0.5)
+                L.up = w((2 if m.act == "silu_gate" else 1) * m.ff, W, std=W ** -0.5)  # silu_gate: the gate rows, then the up rows
                 L.down = w(W, m.ff, std=m.ff ** -0.5)
                 L.act = torch.tensor([0.3, -0.4] if m.act == "xielu" else [1.0, 0.3, 0.1, 0.01], dtype=torch.float32, device=device)
+            if isinstance(m, MoeSpec) and m.shared_ff:
+                L.sh_up = w(2 * m.shared_ff, W, std=W ** -0.5)
+                L.sh_down = w(W, m.shared_ff, std=m.shared_ff ** -0.5)
+            if self.conv_stream:
+                L.norm1, L.norm2 = (1.0 + L.norm1.float()).to(dtype), None if L.norm2 is None else (1.0 + L.norm2.float()).to(dtype)
+                if cfg.conv_taps:
+                    L.canon1 = w(W, cfg.conv_taps, std=0.3)
+                    L.canon2 = w(W, cfg.conv_taps, std=0.3) if m is not None else None
             if self.pre_norm:
                 L.norm1, L.norm2 = (1.0 + L.norm1.float()).to(dtype), None if L.norm2 is None else (1.0 + L.norm2.float()).to(dtype)
                 c = torch.full((len(self.layers) + 2,), 0.1, dtype=torch.float32, device=device)
@@ -425,6 +576,11 @@ class HybridDecoder:
             self.final_norm = (1.0 + self.final_norm.float()).to(dtype)
             self.embed_norm = (1.0 + w(W, std=0.1).float()).to(dtype)
             self.head = w(cfg.vocab_size, W, std=W ** -0.5)
+        if self.conv_stream:
+            self.final_norm = (1.0 + self.final_norm.float()).to(dtype)
+            self.head = w(cfg.vocab_size, W, std=W ** -0.5)
+            if cfg.loop is not None:
+                self.loop_step = f32(cfg.loop[2], W, std=0.3)
         if self.parallel:
             self.final_norm = f32(W, std=0.1)
             self.head = w(cfg.vocab_size, W, std=W ** -0.5)
@@ -443,13 +599,13 @@ class HybridDecoder:
     def _tensors(self):
         yield self.embed
         yield self.final_norm
-        for t in (self.embed_norm, self.head, self.pair_table):
+        for t in (self.embed_norm, self.head, self.pair_table, self.loop_step):
             if t is not None:
                 yield t
         for L in self.layers:
             for k in ("w_in", "o", "norm1", "norm2", "uk_t", "uv", "c_norm", "out_norm", "router", "bias", "up", "down", "talk", "lam",
                       "taps", "rate", "dt_bias", "a2", "g2", "act", "depth_w", "sink", "ls1", "ls2", "shift", "in_bias", "out_bias", "pb",
-                      "skip", "conv_b"):
+                      "skip", "conv_b", "canon1", "canon2", "w_x", "w_dt", "sh_up", "sh_down"):
                 t = getattr(L, k)
                 if t is not None:
                     yield t
@@ -480,10 +636,18 @@ class HybridDecoder:
             put(self.head, state["head"])
             if self.pair_table is not None:
                 put(self.pair_table, state["bigram"])
+        if self.conv_stream:
+            put(self.head, state["head"])
+            if self.loop_step is not None:
+                put(self.loop_step, state["loop.step"])
         for i, L in enumerate(self.layers):
             s, p = L.spec, f"l{i}.mix."
             H, d, dv = s.heads, s.dim, s.vdim
             put(L.norm1, state[f"l{i}.norm1"])
+            if L.canon1 is not None:
+                put(L.canon1, state[f"l{i}.canon1"])
+            if L.canon2 is not None:
+                put(L.canon2, state[f"l{i}.canon2"])
             if L.depth_w is not None:
                 put(L.depth_w, state[f"l{i}.dwa"])
             if self.parallel:
@@ -507,6 +671,17 @@ class HybridDecoder:
                 put(L.out_norm, state[b + "norm"])
                 put(L.o, torch.cat([state[a + "o"], state[b + "o"]], dim=1))
                 put(L.out_bias, state[a + "o.b"])
+            elif s.kind == "mamba1":
+                put(L.w_in, state[p + "in"])
+                put(L.taps, state[p + "conv"])
+                put(L.conv_b, state[p + "conv.b"])
+                put(L.w_x, state[p + "x"])
+                put(L.w_dt, state[p + "dt"])
+                put(L.dt_bias, state[p + "dt.b"])
+                put(L.rate, -torch.exp(state[p + "A_log"].to(torch.float32)))
+                put(L.skip, state[p + "D"])
+            elif s.kind == "sink_attention":
+                put(L.w_in, torch.cat([state[p + "q"], state[p + "k"], state[p + "v"]], dim=0))
             elif s.kind == "attention":
                 put(L.w_in, torch.cat([state[p + "q"], state[p + "k"], state[p + "v"], state[p + "g"]], dim=0))
                 put(L.talk, state[p + "talk"])
@@ -522,7 +697,7 @@ class HybridDecoder:
                     put(L.a2, state[p + "a2"])
                     put(L.g2, state[p + "g2"])
             elif s.kind == "latent_attention":
-                parts = [state[p + "q"]] + ([] if s.kv_from is not None else [state[p + "dkv"]])
+                parts = [state[p + "q"]] + ([] if s.kv_from is not None else [state[p + "dkv"]]) + ([state[p + "g"]] if s.out_gate else [])
                 put(L.w_in, torch.cat(parts, dim=0))
                 put(L.uk_t, state[p + "uk"].view(H, d, s.kv_rank).transpose(1, 2).contiguous())
                 put(L.uv, state[p + "uv"].view(H, dv, s.kv_rank))
@@ -533,10 +708,15 @@ class HybridDecoder:
                 put(L.out_norm, state[p + "norm"])
             if s.kind != "parallel":
                 put(L.o, state[p + "o"])
-            if s.mlp is None and f"l{i}.norm2" in state and not self.pre_norm and not self.parallel:  # no feed-forward, but a second norm
+            if s.mlp is None and f"l{i}.norm2" in state and not self.pre_norm and not self.parallel and not self.conv_stream:  # no feed-forward, but a second norm
                 L.norm2 = torch.empty_like(L.norm1)
                 put(L.norm2, state[f"l{i}.norm2"])
-            if isinstance(s.mlp, DenseFfSpec):
+            if isinstance(s.mlp, DenseFfSpec) and s.mlp.act == "silu_gate":
+                q = f"l{i}.mlp."
+                put(L.norm2, state[f"l{i}.norm2"])
+                put(L.up, torch.cat([state[q + "gate"], state[q + "up"]], dim=0))
+                put(L.down, state[q + "down"])
+            elif isinstance(s.mlp, DenseFfSpec):
                 q = f"l{i}.mlp."
                 if L.norm2 is not None:
                     put(L.norm2, state[f"l{i}.norm2"])
@@ -547,7 +727,13 @@ class HybridDecoder:
                 q = f"l{i}.mlp."
                 put(L.norm2, state[f"l{i}.norm2"])
                 put(L.router, state[q + "router"])
-                put(L.bias, state[q + "router.b"])
+                if s.mlp.pick == "sigmoid_input":
+                    L.bias = None
+                    if s.mlp.shared_ff:
+                        put(L.sh_up, torch.cat([state[q + "shared.gate"], state[q + "shared.up"]], dim=0))
+                        put(L.sh_down, state[q + "shared.down"])
+                else:
+                    put(L.bias, state[q + "router.b"])
                 put(L.up, torch.stack([torch.cat([state[f"{q}e{e}.gate"], state[f"{q}e{e}.up"]], dim=0) for e in range(s.mlp.experts)]))
                 put(L.down, torch.stack([state[f"{q}e{e}.down"] for e in range(s.mlp.experts)]))
             elif s.mlp is not None:
@@ -571,10 +757,18 @@ class HybridDecoder:
             out["head"] = self.head
             if self.pair_table is not None:
                 out["bigram"] = self.pair_table
+        if self.conv_stream:
+            out["head"] = self.head
+            if self.loop_step is not None:
+                out["loop.step"] = self.loop_step
         for i, L in enumerate(self.layers):
             s, p = L.spec, f"l{i}.mix."
             H, d, dv = s.heads, s.dim, s.vdim
             out[f"l{i}.norm1"] = L.norm1
+            if L.canon1 is not None:
+                out[f"l{i}.canon1"] = L.canon1
+            if L.canon2 is not None:
+                out[f"l{i}.canon2"] = L.canon2
             if L.depth_w is not None:
                 out[f"l{i}.dwa"] = L.depth_w
             if self.parallel:
@@ -595,6 +789,11 @@ class HybridDecoder:
                 out[b + "A_log"], out[b + "D"], out[b + "norm"] = torch.log(-L.rate), L.skip, L.out_norm
                 out[a + "o"], out[b + "o"] = L.o[:, : H * dv], L.o[:, H * dv:]
                 out[a + "o.b"] = L.out_bias
+            elif s.kind == "mamba1":
+                out[p + "in"], out[p + "conv"], out[p + "conv.b"], out[p + "x"], out[p + "dt"] = L.w_in, L.taps, L.conv_b, L.w_x, L.w_dt
+                out[p + "dt.b"], out[p + "A_log"], out[p + "D"] = L.dt_bias, torch.log(-L.rate), L.skip
+            elif s.kind == "sink_attention":
+                out[p + "q"], out[p + "k"], out[p + "v"] = torch.split(L.w_in, [H * d, s.kv_heads * d, s.kv_heads * dv], dim=0)
             elif s.kind == "attention":
                 cuts = [H * d, s.kv_heads * d, s.kv_heads * dv, H]
                 out[p + "q"], out[p + "k"], out[p + "v"], out[p + "g"] = torch.split(L.w_in, cuts, dim=0)
@@ -613,7 +812,9 @@ class HybridDecoder:
                 nq = H * (d + s.rot_dim)
                 out[p + "q"] = L.w_in[:nq]
                 if s.kv_from is None:
-                    out[p + "dkv"], out[p + "dkv.norm"] = L.w_in[nq:], L.c_norm
+                    out[p + "dkv"], out[p + "dkv.norm"] = L.w_in[nq: nq + s.kv_rank + s.rot_dim], L.c_norm
+                if s.out_gate:
+                    out[p + "g"] = L.w_in[L.w_in.shape[0] - H * dv:]
                 out[p + "uk"] = L.uk_t.transpose(1, 2).reshape(H * d, s.kv_rank)
                 out[p + "uv"] = L.uv.reshape(H * dv, s.kv_rank)
             else:
@@ -624,14 +825,23 @@ class HybridDecoder:
                 out[p + "o"] = L.o
             if s.mlp is None and L.norm2 is not None:
                 out[f"l{i}.norm2"] = L.norm2
-            if isinstance(s.mlp, DenseFfSpec):
+            if isinstance(s.mlp, DenseFfSpec) and s.mlp.act == "silu_gate":
+                q = f"l{i}.mlp."
+                out[f"l{i}.norm2"], out[q + "gate"], out[q + "up"], out[q + "down"] = L.norm2, L.up[: s.mlp.ff], L.up[s.mlp.ff:], L.down
+            elif isinstance(s.mlp, DenseFfSpec):
                 q = f"l{i}.mlp."
                 out[q + "up"], out[q + "down"], out[q + "act"] = L.up, L.down, L.act
                 if L.norm2 is not None:
                     out[f"l{i}.norm2"] = L.norm2
             elif isinstance(s.mlp, MoeSpec) and s.mlp.gated:
                 q = f"l{i}.mlp."
-                out[f"l{i}.norm2"], out[q + "router"], out[q + "router.b"] = L.norm2, L.router, L.bias
+                out[f"l{i}.norm2"], out[q + "router"] = L.norm2, L.router
+                if s.mlp.pick == "sigmoid_input":
+                    if s.mlp.shared_ff:
+                        out[q + "shared.gate"], out[q + "shared.up"] = L.sh_up[: s.mlp.shared_ff], L.sh_up[s.mlp.shared_ff:]
+                        out[q + "shared.down"] = L.sh_down
+                else:
+                    out[q + "router.b"] = L.bias
                 for e in range(s.mlp.experts):
                     out[f"{q}e{e}.gate"], out[f"{q}e{e}.up"], out[f"{q}e{e}.down"] = L.up[e, : s.mlp.ff], L.up[e, s.mlp.ff:], L.down[e]
             elif s.mlp is not None:
@@ -663,9 +873,112 @@ class HybridDecoder:
         splits = mixops.latent_attn_splits(md.batch, T, H, md.max_seqlen_k) if md.max_seqlen_q <= 16 else 1
         mixops.latent_attn(o_lat, q_abs, rows, ctx.page_table, md.req_rows, md.seq_lens, md.cu_seqlens_q, md.batch, R, s.scale,
                            splits=splits, sink=L.sink)
-        o = torch.empty((T, H * dv), dtype=self.dtype, device=h.device)
+        # with an output gate the heads' values stay fp32 until the gate has multiplied them: one rounding on the way into W_o
+        o = torch.empty((T, H * dv), dtype=torch.float32 if s.out_gate else self.dtype, device=h.device)
         mixops.gemm_nt(o, o_lat, L.uv, T, dv, R, lda=H * R, ldb=R, ldc=H * dv, groups=H, a_gs=R, b_gs=dv * R, c_gs=dv)
+        if s.out_gate:
+            g_off = L.w_in.shape[0] - H * dv
+            o = mixops.sigmoid_gate(o, proj[:, g_off:])
         return mixops.linear(o, L.o)
+
+    def _mamba(self, i: int, L: _Layer, h: torch.Tensor, ctx: Any, batch: Any) -> torch.Tensor:
+        """Selective scan: in-projection, causal convolution + SiLU with the request's conv state, the two-step step-size projection,
+        the recurrence on the request's fp32 state (gated by silu(z) in the same launch), output projection."""
+        s, md, kv = L.spec, batch.attn_metadata, ctx.kv_cache
+        inner, N, dr = s.vdim, s.dim, s.dt_rank
+        proj = mixops.linear(h, L.w_in)
+        x = mixops.short_conv(proj, inner, L.taps, kv.conv_state(i), md.cu_seqlens_q, md.seq_lens, md.req_rows, md.batch, unit_heads=0,
+                              scaled_heads=0, d=1, bias=L.conv_b, model_dtype=True)
+        dbc = mixops.linear(x, L.w_x)
+        dt_in = mixops.linear(dbc[:, :dr], L.w_dt)
+        y = mixops.selective_scan(x, proj[:, inner:], dt_in, dbc[:, dr:], L.rate, L.dt_bias, L.skip, kv.state(i), md.cu_seqlens_q, md.seq_lens,
+                                  md.req_rows, md.batch, chunks=getattr(md, "scan_chunks", None))
+        return mixops.linear(y, L.o)
+
+    def _sink_attention(self, i: int, L: _Layer, h: torch.Tensor, ctx: Any, batch: Any) -> torch.Tensor:
+        """Grouped attention over a window with a sink: projections, rotation of q and k and unit-RMS values into the cache rows, scores /
+        softmax / weighted values in one launch, output projection."""
+        s, md, kv = L.spec, batch.attn_metadata, ctx.kv_cache
+        T, H, G, d, dv = h.shape[0], s.heads, s.kv_heads, s.dim, s.vdim
+        proj = mixops.linear(h, L.w_in)
+        kc, vc = kv.kv_rows(i)
+        q = mixops.qk_prep(proj, None, kc, vc, batch.out_loc, batch.positions, L.cos_sin, self.cfg.rms_norm_eps, H, G, d, dv,
+                           interleaved=False, unit=False, unit_v=s.v_norm)
+        o = torch.empty((T, H * dv), dtype=self.dtype, device=h.device)
+        splits = mixops.sink_attn_splits(md.batch, T, H, G, s.window, md.max_seqlen_k) if md.max_seqlen_q <= 16 else 1
+        mixops.sink_attn(o, q, kc, vc, ctx.page_table, md.req_rows, md.seq_lens, md.cu_seqlens_q, md.batch, H, G, d, dv, s.scale, s.window,
+                         L.sink if s.sink else None, splits=splits)
+        return mixops.linear(o, L.o)
+
+    def _gated_ff(self, h: torch.Tensor, up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:
+        return mixops.linear(mixops.silu_mul(mixops.linear(h, up)), down)
+
+    def _input_weighted_experts(self, L: _Layer, h: torch.Tensor) -> torch.Tensor:
+        """-> [T, top, W]: every chosen expert's output on score * h (the score is inside the expert's input, so the caller adds the
+        rows as they are)."""
+        m, (T, W) = L.spec.mlp, h.shape
+        ids, wts = mixops.route_sigmoid(h, L.router, m.top)
+        hs = mixops.scale_rows(h, wts)
+        seg, perm = mixops.moe_sort(ids, m.experts)
+        n = T * m.top
+        gu = torch.empty((n, 2 * m.ff), dtype=self.dtype, device=h.device)
+        mixops.gemm_nt(gu, hs, L.up, n, 2 * m.ff, W, lda=W, ldb=W, ldc=2 * m.ff, groups=m.experts, b_gs=2 * m.ff * W, seg=seg, a_rows=perm, a_div=1)
+        act = mixops.silu_mul(gu)
+        y = torch.empty((T, m.top, W), dtype=self.dtype, device=h.device)
+        mixops.gemm_nt(y, act, L.down, n, W, m.ff, lda=m.ff, ldb=m.ff, ldc=W, groups=m.experts, b_gs=W * m.ff, seg=seg, c_rows=perm)
+        return y
+
+    def _forward_conv(self, ctx: Any, batch: Any, layer_outputs: Optional[list]) -> torch.Tensor:
+        """The pre-norm stream with grouped norms, input convolutions and a looped run of layers -> the final-normed rows [tokens, W].
+        One `norm_conv` launch closes a sublayer (residual sum with the multiplier, the loop's step vector) and opens the next (norm,
+        input convolution); the convolutions' new state rows are staged and committed after the last layer."""
+        cfg, eps, md, kv = self.cfg, self.cfg.rms_norm_eps, batch.attn_metadata, ctx.kv_cache
+        T, W, dev, bs = batch.input_ids.shape[0], cfg.hidden_size, self.device, batch.attn_metadata.batch
+        runs, n, mult, groups = cfg.runs, cfg.conv_taps, cfg.residual_mult, cfg.norm_groups
+        req = dict(cu_q=md.cu_seqlens_q, seq_lens=md.seq_lens, req_rows=md.req_rows, batch=bs)
+        staging = torch.empty((len(runs), 2, bs, n - 1, W), dtype=torch.float32, device=dev) if n > 1 else None
+        x = mixops.embed_scaled(self.embed, batch.input_ids, 1.0)
+
+        def open_sublayer(x_in, parts, add, weight, taps, run, sub):
+            """-> (x after the sum, the sublayer's input rows in the model dtype)."""
+            h = torch.empty((T, W), dtype=self.dtype, device=dev)
+            x_out = torch.empty((T, W), dtype=torch.float32, device=dev) if parts or add is not None else None
+            conv = dict(taps=taps, state=kv.conv_in_state(run, sub), staging=staging[run, sub], **req) if taps is not None and n > 1 else dict(taps=taps)
+            mixops.norm_conv(x_in, weight, eps, groups, h, parts=parts, mult=mult, add=add, x_out=x_out, **conv)
+            return (x_in if x_out is None else x_out), h
+
+        pending: tuple = ()
+        for run, (i, pass_no) in enumerate(runs):
+            L = self.layers[i]
+            add = self.loop_step[pass_no] if pass_no is not None else None
+            x, h = open_sublayer(x, pending, add, L.norm1, L.canon1, run, 0)
+            if layer_outputs is not None and run > 0:
+                layer_outputs.append(x - add if add is not None else x.clone())
+            kind = L.spec.kind
+            if kind == "latent_attention":
+                y = self._latent(run, L, h, ctx, batch)
+            elif kind == "mamba1":
+                y = self._mamba(run, L, h, ctx, batch)
+            elif kind == "sink_attention":
+                y = self._sink_attention(run, L, h, ctx, batch)
+            else:
+                raise NotImplementedError(f"mixer {kind!r} in a looped pre-norm stack")
+            m = L.spec.mlp
+            if m is None:
+                pending = (y,)
+                continue
+            x, h = open_sublayer(x, (y,), None, L.norm2, L.canon2, run, 1)
+            if isinstance(m, DenseFfSpec):
+                pending = (self._gated_ff(h, L.up, L.down),)
+            else:
+                pending = (self._input_weighted_experts(L, h),) + ((self._gated_ff(h, L.sh_up, L.sh_down),) if m.shared_ff else ())
+        x, hf = open_sublayer(x, pending, None, self.final_norm, None, 0, 0)
+        if layer_outputs is not None and runs:
+            layer_outputs.append(x.clone())
+        if staging is not None:
+            mixops.commit_rows(kv.conv_in_states.view(2 * len(runs), -1, (n - 1) * W), staging.view(2 * len(runs), bs, (n - 1) * W), md.req_rows, bs,
+                               md.cu_seqlens_q)
+        return hf
 
     def _lightning(self, i: int, L: _Layer, h: torch.Tensor, ctx: Any, batch: Any) -> torch.Tensor:
         s, md = L.spec, batch.attn_metadata
@@ -856,16 +1169,19 @@ class HybridDecoder:
         last token (prefill) or at every token (decode)."""
         cfg = self.cfg
         eps, alpha = cfg.rms_norm_eps, cfg.postln_alpha
-        if self.pre_norm or self.parallel:
-            hf = self._forward_pre_norm(ctx, batch, layer_outputs) if self.pre_norm else self._forward_parallel(ctx, batch, layer_outputs)
+        if self.pre_norm or self.parallel or self.conv_stream:
+            hf = self._forward_pre_norm(ctx, batch, layer_outputs) if self.pre_norm else \
+                self._forward_parallel(ctx, batch, layer_outputs) if self.parallel else self._forward_conv(ctx, batch, layer_outputs)
             rows = getattr(batch, "logit_rows", None)
             if rows is None and batch.is_prefill:
                 rows = batch.attn_metadata.get_last_indices(batch.size)
             if rows is not None:
                 hf = hf.index_select(0, rows.to(torch.int64))
             if logits_out is not None and logits_out.shape == (hf.shape[0], cfg.vocab_size) and logits_out.dtype == self.dtype:
-                return mixops.linear(hf, self.head, out=logits_out)
-            return mixops.linear(hf, self.head)
+                logits = mixops.linear(hf, self.head, out=logits_out)
+            else:
+                logits = mixops.linear(hf, self.head)
+            return mixops.softcap(logits, cfg.logit_softcap) if cfg.logit_softcap > 0.0 else logits
         x, h = mixops.embed(self.embed, batch.input_ids)
         for i, L in enumerate(self.layers):
             y = self._latent(i, L, h, ctx, batch) if L.spec.kind == "latent_attention" else self._lightning(i, L, h, ctx, batch)

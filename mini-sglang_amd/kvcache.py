@@ -80,9 +80,11 @@ def create_kvcache_pool(model_config, num_pages: int, page_size: int, dtype: tor
     """P/kvcache/__init__.py:27-44; a configuration that lists its layers one by one (`layers` of specs) gets the per-layer
     HybridCache with `state_rows` recurrent-state slots."""
     if hasattr(model_config, "layers"):
-        return HybridCache(model_config.layers, num_pages, page_size, state_rows, dtype, device,
+        # a configuration with a repeated run of layers lists one spec per layer RUN (`cache_layers`): every pass has its own rows
+        return HybridCache(getattr(model_config, "cache_layers", model_config.layers), num_pages, page_size, state_rows, dtype, device,
                            shift_width=model_config.hidden_size if getattr(model_config, "token_shift", False) else 0,
-                           prev_token=getattr(model_config, "pair_embed", None) is not None)
+                           prev_token=getattr(model_config, "pair_embed", None) is not None,
+                           conv_in=(getattr(model_config, "conv_taps", 0), model_config.hidden_size))
     return MHAKVCache(num_kv_heads=model_config.num_kv_heads, num_pages=num_pages, page_size=page_size,
                       num_layers=model_config.num_layers, head_dim=model_config.head_dim, device=device,
                       dtype=dtype, tp_size=tp_size)
@@ -110,14 +112,24 @@ class HybridCache:
       request, the last normed row in fp32: `shift_state(layer)` is `[state_rows, width]` (all layers: `shift_states`);
     * a model whose embedding depends on the previous token (`prev_token`) keeps each request's last token id: `prev_token`,
       int32 `[state_rows]`.
+    * a windowed attention layer with a sink (`sink_attention`) caches keys and (normed) values like `attention`: every token stays
+      cached, the window is applied when reading;
+    * a selective-scan layer (`mamba1`) keeps the fp32 state `[state_rows, inner, state]` and the last `conv - 1` inputs of its
+      convolution, `conv_state(layer)` = `[state_rows, conv - 1, inner]` in the model dtype;
+    * a model with a causal convolution of `taps` in front of every sublayer (`conv_in` = (taps, width)) keeps, per layer, sublayer and
+      request, the last `taps - 1` normed rows in fp32: `conv_in_state(layer, sub)` is `[state_rows, taps - 1, width]` (all of them:
+      `conv_in_states`, `[layers, 2, state_rows, taps - 1, width]`).
     Layers may differ in every size, so each gets its own allocation.  Every per-request row is indexed by the request's
     page-table row and needs no clearing: a request whose first token is at position 0 never reads what the row held.
     """
 
     def __init__(self, layers, num_pages: int, page_size: int, state_rows: int, dtype: torch.dtype, device: torch.device,
-                 shift_width: int = 0, prev_token: bool = False) -> None:
+                 shift_width: int = 0, prev_token: bool = False, conv_in=(0, 0)) -> None:
         self._latent, self._state, self._owner, self._kv, self._conv = {}, {}, {}, {}, {}
         slots = num_pages * page_size
+        taps_in, width_in = conv_in
+        self.conv_in_states = torch.zeros((len(layers), 2, state_rows, taps_in - 1, width_in), dtype=torch.float32, device=device) \
+            if taps_in > 1 else None
         self.shift_states = torch.zeros((len(layers), state_rows, shift_width), dtype=torch.float32, device=device) if shift_width else None
         self.prev_token = torch.zeros((state_rows,), dtype=torch.int32, device=device) if prev_token else None
         for i, spec in enumerate(layers):
@@ -134,9 +146,13 @@ class HybridCache:
                 self._owner[i] = i if spec.kv_from is None else spec.kv_from
             elif spec.kind == "lightning":
                 self._state[i] = torch.zeros((state_rows, spec.heads, spec.dim, spec.vdim), dtype=torch.float32, device=device)
-            elif spec.kind == "attention":
+            elif spec.kind in ("attention", "sink_attention"):
                 self._kv[i] = (torch.zeros((slots, spec.kv_heads * spec.dim), dtype=dtype, device=device),
                                torch.zeros((slots, spec.kv_heads * spec.vdim), dtype=dtype, device=device))
+            elif spec.kind == "mamba1":
+                self._state[i] = torch.zeros((state_rows, spec.vdim, spec.dim), dtype=torch.float32, device=device)
+                if spec.conv > 1:
+                    self._conv[i] = torch.zeros((state_rows, spec.conv - 1, spec.vdim), dtype=dtype, device=device)
             elif spec.kind in ("delta", "channel_delta"):
                 self._state[i] = torch.zeros((state_rows, spec.heads, spec.dim, spec.vdim), dtype=torch.float32, device=device)
                 if spec.conv > 1:
@@ -166,6 +182,10 @@ class HybridCache:
         """[state_rows, conv - 1, channels] of a delta-rule or state-space layer, or None when its convolution has one tap."""
         return self._conv.get(layer)
 
+    def conv_in_state(self, layer: int, sub: int) -> torch.Tensor:
+        """fp32 [state_rows, taps - 1, width]: every request's last normed rows in front of sublayer `sub` (0 mixer, 1 feed-forward)."""
+        return self.conv_in_states[layer, sub]
+
     def shift_state(self, layer: int) -> torch.Tensor:
         """fp32 [state_rows, width]: every request's last normed row of this layer."""
         return self.shift_states[layer]
@@ -174,18 +194,21 @@ class HybridCache:
     def bytes_per_page(layers, page_size: int, dtype: torch.dtype) -> int:
         es = torch.empty((), dtype=dtype).element_size()
         per_token = sum(s.kv_rank + s.rot_dim for s in layers if s.kind == "latent_attention" and s.kv_from is None)
-        per_token += sum(s.kv_heads * (s.dim + s.vdim) for s in layers if s.kind == "attention")
+        per_token += sum(s.kv_heads * (s.dim + s.vdim) for s in layers if s.kind in ("attention", "sink_attention"))
         per_token += sum(s.left.kv_heads * (s.left.dim + s.left.vdim) for s in layers if s.kind == "parallel")
         return per_token * es * page_size
 
     @staticmethod
-    def state_bytes(layers, state_rows: int, dtype: torch.dtype = torch.bfloat16, shift_width: int = 0) -> int:
+    def state_bytes(layers, state_rows: int, dtype: torch.dtype = torch.bfloat16, shift_width: int = 0, conv_in=(0, 0)) -> int:
         es = torch.empty((), dtype=dtype).element_size()
+        taps_in, width_in = conv_in
         total = sum(4 * s.heads * s.dim * s.vdim * state_rows for s in layers if s.kind in ("lightning", "delta", "channel_delta"))
         total += sum(es * (s.conv - 1) * (2 * s.kv_heads * s.dim + s.heads * s.vdim) * state_rows
                      for s in layers if s.kind in ("delta", "channel_delta"))
         for s in (x.right for x in layers if x.kind == "parallel"):
             total += (4 * s.heads * s.dim * s.vdim + es * (s.conv - 1) * (s.heads * s.vdim + 2 * s.kv_heads * s.dim)) * state_rows
+        total += sum((4 * s.vdim * s.dim + es * (s.conv - 1) * s.vdim) * state_rows for s in layers if s.kind == "mamba1")
+        total += 4 * 2 * max(taps_in - 1, 0) * width_in * len(layers) * state_rows
         return total + 4 * shift_width * len(layers) * state_rows
 
     @property

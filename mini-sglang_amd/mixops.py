@@ -387,17 +387,19 @@ def window_attn(out: torch.Tensor, src: torch.Tensor, g_off: int, k_cache: torch
 
 
 def short_conv(src: torch.Tensor, C: int, taps: torch.Tensor, state: Optional[torch.Tensor], cu_q: torch.Tensor, seq_lens: torch.Tensor,
-               slots: torch.Tensor, batch: int, unit_heads: int, scaled_heads: int, d: int, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+               slots: torch.Tensor, batch: int, unit_heads: int, scaled_heads: int, d: int, bias: Optional[torch.Tensor] = None,
+               model_dtype: bool = False) -> torch.Tensor:
     """Causal per-channel convolution + SiLU of src[:, :C] (taps [C, n]; state [slots, n - 1, C] carries the inputs before the
-    portion and is moved on), unit vectors for the first `unit_heads` groups of d channels -> fp32 [T, C]."""
+    portion and is moved on), unit vectors for the first `unit_heads` groups of d channels -> fp32 [T, C] (model_dtype: in src's
+    dtype instead, for a result that feeds a projection)."""
     _dev(src, taps, state, cu_q, seq_lens, slots, bias)
     T, n = src.shape[0], taps.shape[1]
     assert bias is None or (bias.dtype == src.dtype and bias.shape == (C,) and bias.is_contiguous())
     assert src.stride(1) == 1 and taps.is_contiguous() and taps.shape[0] == C and taps.dtype == src.dtype
     assert n == 1 or (state.is_contiguous() and state.dtype == src.dtype and state.shape[1:] == (n - 1, C))
-    out = torch.empty((T, C), dtype=torch.float32, device=src.device)
+    out = torch.empty((T, C), dtype=src.dtype if model_dtype else torch.float32, device=src.device)
     check_mix(mix_lib().msgl_mix_short_conv(
-        out.data_ptr(), src.data_ptr(), src.stride(0), taps.data_ptr(), _p(bias), _p(state), _i32(cu_q).data_ptr(), _i32(seq_lens).data_ptr(),
+        0 if model_dtype else out.data_ptr(), out.data_ptr() if model_dtype else 0, src.data_ptr(), src.stride(0), taps.data_ptr(), _p(bias), _p(state), _i32(cu_q).data_ptr(), _i32(seq_lens).data_ptr(),
         _i32(slots).data_ptr(), batch, T, C, n, unit_heads, scaled_heads, d, _code(src), _stream()), "short_conv")
     return out
 
@@ -512,8 +514,9 @@ def commit_rows(dst: Optional[torch.Tensor], src: Optional[torch.Tensor], slots:
 
 def qk_prep(proj: torch.Tensor, bias: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: torch.Tensor, out_loc: torch.Tensor,
             positions: torch.Tensor, cos_sin: Optional[torch.Tensor], eps: float, H: int, G: int, d: int, dv: int, *, interleaved: bool,
-            unit: bool) -> torch.Tensor:
-    """Projection rows [q | k | v | ...] (+ fp32 bias) -> rotated (and unit-RMS) q as fp32 [T, H * d]; k, v into the cache rows."""
+            unit: bool, unit_v: bool = False) -> torch.Tensor:
+    """Projection rows [q | k | v | ...] (+ fp32 bias) -> rotated (and unit-RMS) q as fp32 [T, H * d]; k, v into the cache rows
+    (unit_v: every value head divided by its root mean square first)."""
     _dev(proj, bias, k_cache, v_cache, out_loc, positions, cos_sin)
     T = proj.shape[0]
     n = (H + G) * d + G * dv
@@ -527,7 +530,7 @@ def qk_prep(proj: torch.Tensor, bias: Optional[torch.Tensor], k_cache: torch.Ten
     q = torch.empty((T, H * d), dtype=torch.float32, device=proj.device)
     check_mix(mix_lib().msgl_mix_qk_prep(
         proj.data_ptr(), proj.stride(0), _p(bias), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _i32(out_loc).data_ptr(),
-        _i32(positions).data_ptr(), _p(cos_sin), rd, int(interleaved), int(unit), float(eps), T, H, G, d, dv, _code(proj), _stream()),
+        _i32(positions).data_ptr(), _p(cos_sin), rd, int(interleaved), int(unit) | (2 if unit_v else 0), float(eps), T, H, G, d, dv, _code(proj), _stream()),
         "qk_prep")
     return q
 
@@ -608,3 +611,151 @@ def xielu(z: torch.Tensor, pq: torch.Tensor) -> torch.Tensor:
     out = torch.empty((rows, N), dtype=z.dtype, device=z.device)
     check_mix(mix_lib().msgl_mix_xielu(out.data_ptr(), z.data_ptr(), z.stride(0), pq.data_ptr(), rows, N, _code(z), _stream()), "xielu")
     return out
+
+
+# ------------------------------------------------------------------ looped pre-norm hybrid decoders (csrc/mix_scan.hip)
+def norm_conv(x: torch.Tensor, weight: torch.Tensor, eps: float, groups: int, h_out: torch.Tensor, *, parts=(), mult: float = 1.0,
+              add: Optional[torch.Tensor] = None, x_out: Optional[torch.Tensor] = None, taps: Optional[torch.Tensor] = None,
+              state: Optional[torch.Tensor] = None, staging: Optional[torch.Tensor] = None, cu_q: Optional[torch.Tensor] = None,
+              seq_lens: Optional[torch.Tensor] = None, req_rows: Optional[torch.Tensor] = None, batch: int = 0) -> None:
+    """row = x + mult * (sum of the parts' rows) + add -> x_out (fp32, a buffer other than x);  h = row normed in `groups` equal parts,
+    times weight;  h_out = h + sum_j taps[:, j] * h of the token (n - 1 - j) before (taps [W, n] in h_out's dtype; the tokens before a
+    portion: state[req_rows[b]], fp32 [rows, n - 1, W]; every request's new state rows -> staging[b], fp32 [batch, n - 1, W]).
+    parts: up to two tensors [rows, W] or [rows, p, W] in h_out's dtype; add: fp32 [W]."""
+    rows, W = x.shape
+    _dev(x, weight, h_out, add, x_out, taps, state, staging, cu_q, seq_lens, req_rows)
+    dt = h_out.dtype
+    assert x.dtype == torch.float32 and x.is_contiguous() and weight.dtype == dt and weight.shape == (W,) and weight.is_contiguous()
+    assert h_out.shape == (rows, W) and h_out.is_contiguous() and len(parts) <= 2 and W % groups == 0
+    _f32(add, W)
+    assert x_out is None or (x_out.dtype == torch.float32 and x_out.is_contiguous() and x_out.shape == (rows, W) and x_out.data_ptr() != x.data_ptr())
+    ys = []
+    for y in parts:
+        _dev(y)
+        assert y.dtype == dt and y.is_contiguous() and y.shape[0] == rows and y.shape[-1] == W and y.dim() in (2, 3)
+        ys.append((y.data_ptr(), 1 if y.dim() == 2 else y.shape[1]))
+    ys += [(0, 0)] * (2 - len(ys))
+    n = 1
+    if taps is not None:
+        n = taps.shape[1]
+        assert taps.dtype == dt and taps.is_contiguous() and taps.shape == (W, n)
+    if n > 1:
+        assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (n - 1, W)
+        assert staging.dtype == torch.float32 and staging.is_contiguous() and staging.shape == (batch, n - 1, W)
+        assert cu_q.numel() >= batch + 1 and seq_lens.numel() >= batch and req_rows.numel() >= batch
+    if rows:
+        check_mix(mix_lib().msgl_mix_norm_conv(
+            x.data_ptr(), _p(x_out), ys[0][0], ys[0][1], ys[1][0], ys[1][1], float(mult), _p(add), weight.data_ptr(), groups, float(eps),
+            _p(taps), n, _p(state) if n > 1 else 0, _p(staging) if n > 1 else 0, h_out.data_ptr(),
+            _p(None if cu_q is None or n == 1 else _i32(cu_q)), _p(None if n == 1 else _i32(seq_lens)), _p(None if n == 1 else _i32(req_rows)),
+            batch, rows, W, _code(h_out), _stream()), "norm_conv")
+
+
+def selective_scan(x: torch.Tensor, z: torch.Tensor, dt_in: torch.Tensor, bc: torch.Tensor, A: torch.Tensor, dt_bias: torch.Tensor,
+                   D: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor, slots: torch.Tensor, batch: int,
+                   chunks=None) -> torch.Tensor:
+    """state: fp32 [slots, C, N]; x, z, dt_in: [T, C] in the model dtype (views with a row stride are fine); bc: [T, 2 N] = B | C;
+    A = -exp(A_log) fp32 [C, N]; dt_bias, D fp32 [C] -> y * silu(z), [T, C] in the model dtype.  chunks = (items int32 [n, 3],
+    item_first int32 [batch + 1], n) cuts long portions into pieces that run in parallel."""
+    _dev(x, z, dt_in, bc, A, dt_bias, D, state, cu_q, seq_lens, slots)
+    _, C, N = state.shape
+    T = x.shape[0]
+    assert state.dtype == torch.float32 and state.is_contiguous() and A.dtype == torch.float32 and A.is_contiguous() and A.shape == (C, N)
+    for t in (x, z, dt_in):
+        assert t.shape == (T, C) and t.stride(1) == 1 and t.dtype == x.dtype
+    assert bc.shape == (T, 2 * N) and bc.stride(1) == 1 and bc.dtype == x.dtype
+    _f32(dt_bias, C), _f32(D, C)
+    out = torch.empty((T, C), dtype=x.dtype, device=x.device)
+    items = first = scratch = None
+    n_items = 0
+    if chunks is not None:
+        items, first, n_items = chunks
+        _dev(items, first)
+        assert items.numel() == 3 * n_items and first.numel() == batch + 1
+        scratch = torch.empty(n_items * C * (N + 1), dtype=torch.float32, device=x.device)
+    check_mix(mix_lib().msgl_mix_selective_scan(
+        out.data_ptr(), x.data_ptr(), x.stride(0), z.data_ptr(), z.stride(0), dt_in.data_ptr(), dt_in.stride(0), bc.data_ptr(), bc.stride(0),
+        A.data_ptr(), dt_bias.data_ptr(), D.data_ptr(), state.data_ptr(), _i32(cu_q).data_ptr(), _i32(seq_lens).data_ptr(),
+        _i32(slots).data_ptr(), batch, C, N, _code(x), n_items, _p(None if items is None else _i32(items)),
+        _p(None if first is None else _i32(first)), _p(scratch), _stream()), "selective_scan")
+    return out
+
+
+def sink_attn_splits(batch: int, total_q: int, H: int, G: int, window: int, max_keys: int) -> int:
+    """Key ranges per request for a step with few query rows: enough workgroups to fill the chip, at least 256 keys each.  A
+    function of static sizes only (batch, rows, the window or the LONGEST possible key count), so a captured graph keeps its grid."""
+    rep = H // G
+    hb = 1
+    while hb * 2 <= min(rep, 64):
+        hb *= 2
+    blocks = (-(-total_q // (64 // hb)) + batch) * G * -(-rep // hb)
+    keys = min(window, max_keys) if window > 0 else max_keys
+    return max(1, min(1024 // max(blocks, 1), keys // 256, 64))
+
+
+def sink_attn(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, table: torch.Tensor, req_rows: torch.Tensor,
+              seq_lens: torch.Tensor, cu_q: torch.Tensor, batch: int, H: int, G: int, d: int, dv: int, scale: float, window: int,
+              sink: Optional[torch.Tensor], splits: int = 1) -> None:
+    """out[:, : H * dv] = softmax attention over the last `window` keys (0: all earlier keys) with exp(sink[h]) as one more term of
+    the denominator (sink fp32 [H] or None)."""
+    _dev(out, q, k_cache, v_cache, table, req_rows, seq_lens, cu_q, sink)
+    T = q.shape[0]
+    assert q.dtype == torch.float32 and q.is_contiguous() and q.shape == (T, H * d)
+    assert out.shape == (T, H * dv) and out.stride(1) == 1 and out.dtype == k_cache.dtype == v_cache.dtype
+    assert k_cache.is_contiguous() and k_cache.shape[1] == G * d and v_cache.is_contiguous() and v_cache.shape[1] == G * dv
+    assert table.dtype == torch.int32 and table.stride(1) == 1 and (sink is None or _f32(sink, H) is not None)
+    assert req_rows.numel() >= batch and seq_lens.numel() >= batch and cu_q.numel() >= batch + 1
+    ws = None
+    if splits > 1:
+        ws = torch.empty(mix_lib().msgl_mix_sink_attn_workspace_floats(T, H, dv, splits), dtype=torch.float32, device=out.device)
+    check_mix(mix_lib().msgl_mix_sink_attn(
+        out.data_ptr(), out.stride(0), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), table.data_ptr(), table.stride(0),
+        _i32(req_rows).data_ptr(), _i32(seq_lens).data_ptr(), _i32(cu_q).data_ptr(), batch, T, H, G, d, dv, float(scale), int(window),
+        _p(sink), _code(k_cache), splits, _p(ws), _stream()), "sink_attn")
+
+
+def route_sigmoid(h: torch.Tensor, router: torch.Tensor, top: int):
+    """-> (expert ids int32 [T, top], weights fp32 [T, top]): fp32 logits (product kernel, fp32 accumulation), the `top` largest
+    win, the weight of a choice is the sigmoid of its logit."""
+    _dev(h, router)
+    T, W = h.shape
+    E = router.shape[0]
+    assert h.is_contiguous() and router.is_contiguous() and router.shape == (E, W) and router.dtype == h.dtype
+    z = torch.empty((T, E), dtype=torch.float32, device=h.device)
+    gemm_nt(z, h, router, T, E, W, lda=W, ldb=W, ldc=E)
+    ids = torch.empty((T, top), dtype=torch.int32, device=h.device)
+    wts = torch.empty((T, top), dtype=torch.float32, device=h.device)
+    check_mix(mix_lib().msgl_mix_route_sigmoid(ids.data_ptr(), wts.data_ptr(), z.data_ptr(), T, E, top, _stream()), "route_sigmoid")
+    return ids, wts
+
+
+def scale_rows(h: torch.Tensor, wts: torch.Tensor) -> torch.Tensor:
+    """-> [T * top, W]: row t * top + k = wts[t, k] * h[t]."""
+    _dev(h, wts)
+    T, W = h.shape
+    top = wts.shape[1]
+    assert h.is_contiguous() and wts.dtype == torch.float32 and wts.is_contiguous() and wts.shape == (T, top)
+    out = torch.empty((T * top, W), dtype=h.dtype, device=h.device)
+    check_mix(mix_lib().msgl_mix_scale_rows(out.data_ptr(), h.data_ptr(), wts.data_ptr(), T, top, W, _code(h), _stream()), "scale_rows")
+    return out
+
+
+def sigmoid_gate(o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+    """-> o * sigmoid(g) in g's dtype; o fp32 [rows, N], g a [rows, N] view with a row stride."""
+    _dev(o, g)
+    rows, N = o.shape
+    assert o.dtype == torch.float32 and o.is_contiguous() and g.shape == (rows, N) and g.stride(1) == 1
+    out = torch.empty((rows, N), dtype=g.dtype, device=o.device)
+    check_mix(mix_lib().msgl_mix_sigmoid_gate(out.data_ptr(), o.data_ptr(), g.data_ptr(), g.stride(0), rows, N, _code(g), _stream()),
+              "sigmoid_gate")
+    return out
+
+
+def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x <- cap * tanh(x / cap) in place."""
+    _dev(x)
+    assert x.dim() == 2 and x.stride(1) == 1
+    if x.shape[0] == 0:
+        return x
+    check_mix(mix_lib().msgl_mix_softcap(x.data_ptr(), x.stride(0), x.shape[0], x.shape[1], float(cap), _code(x), _stream()), "softcap")
+    return x

@@ -10,7 +10,7 @@ import json
 from pathlib import Path
 from typing import Any, Callable, Dict, Tuple
 
-from .hybrid import HybridConfig, HybridDecoder, bedarax_config, givavik_config
+from .hybrid import HybridConfig, HybridDecoder, bedarax_config, givavik_config, piladra_config
 from .model import DenseDecoder, ModelConfig
 
 
@@ -40,6 +40,7 @@ ARCHITECTURES: Dict[str, Tuple[Callable[[Dict[str, Any]], Any], type, Callable[[
     "Nidorax": (HybridConfig.from_json, HybridDecoder, _load_hybrid),
     "Bedarax": (bedarax_config, HybridDecoder, _load_hybrid),
     "Givavik": (givavik_config, HybridDecoder, _load_hybrid),
+    "Piladra": (piladra_config, HybridDecoder, _load_hybrid),
     "Qwen3ForCausalLM": (dense_config_from_hf, DenseDecoder, _load_dense),
     "Qwen2ForCausalLM": (dense_config_from_hf, DenseDecoder, _load_dense),
     "LlamaForCausalLM": (dense_config_from_hf, DenseDecoder, _load_dense),
