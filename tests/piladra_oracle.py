@@ -108,22 +108,46 @@ def latent_attention(h: torch.Tensor, st: Dict[str, torch.Tensor], p: str, m: Di
     return gated @ _w(st, p + "o").T
 
 
+def selective_scan(x: torch.Tensor, dt: torch.Tensor, A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, D: torch.Tensor,
+                   S0: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """x, dt [T, channels]; A [channels, N]; B, C [T, N]; D [channels] -> (y [T, channels], the state after the last token)."""
+    T, ch = x.shape
+    S = torch.zeros(ch, A.shape[1], dtype=F64) if S0 is None else S0.clone()
+    y = torch.zeros(T, ch, dtype=F64)
+    for t in range(T):
+        S = torch.exp(dt[t][:, None] * A) * S + (dt[t] * x[t])[:, None] * B[t][None, :]
+        y[t] = S @ C[t] + D * x[t]
+    return y, S
+
+
 def mamba1(h: torch.Tensor, st: Dict[str, torch.Tensor], p: str, m: Dict[str, Any]) -> torch.Tensor:
-    T = h.shape[0]
     inner, N, dr = int(m["inner"]), int(m["state"]), int(m["dt_rank"])
     xz = h @ _w(st, p + "in").T
     x, z = xz[:, :inner], xz[:, inner:]
     x = silu(causal_taps(x, _w(st, p + "conv")) + _w(st, p + "conv.b"))
     dbc = x @ _w(st, p + "x").T
     dt = softplus(dbc[:, :dr] @ _w(st, p + "dt").T + _w(st, p + "dt.b"))
-    B, C = dbc[:, dr: dr + N], dbc[:, dr + N: dr + 2 * N]
-    A = -torch.exp(_w(st, p + "A_log"))
-    S = torch.zeros(inner, N, dtype=F64)
-    y = torch.zeros(T, inner, dtype=F64)
-    for t in range(T):
-        S = torch.exp(dt[t][:, None] * A) * S + (dt[t] * x[t])[:, None] * B[t][None, :]
-        y[t] = S @ C[t] + _w(st, p + "D") * x[t]
+    y, _ = selective_scan(x, dt, -torch.exp(_w(st, p + "A_log")), dbc[:, dr: dr + N], dbc[:, dr + N: dr + 2 * N], _w(st, p + "D"))
     return (y * silu(z)) @ _w(st, p + "o").T
+
+
+def windowed_sink_softmax(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, window: int,
+                          sink: Optional[torch.Tensor]) -> torch.Tensor:
+    """q [T, H, d], k [T, G, d], v [T, G, dv] -> [T, H, dv]: token i weighs the keys j with 0 <= i - j < window (window 0: all j <= i)
+    by exp(score) over the sum of these and exp(sink[h])."""
+    T, H, _ = q.shape
+    G, dv = k.shape[1], v.shape[2]
+    out = torch.zeros(T, H, dv, dtype=F64)
+    for i in range(T):
+        lo = max(0, i - window + 1) if window > 0 else 0
+        for hh in range(H):
+            g = hh // (H // G)
+            s = (k[lo: i + 1, g] @ q[i, hh]) * scale
+            mx = s.max() if sink is None else torch.maximum(s.max(), sink[hh])
+            e = torch.exp(s - mx)
+            den = e.sum() + (torch.exp(sink[hh] - mx) if sink is not None else 0.0)
+            out[i, hh] = (e / den) @ v[lo: i + 1, g]
+    return out
 
 
 def window_attention(h: torch.Tensor, st: Dict[str, torch.Tensor], p: str, m: Dict[str, Any], eps: float) -> torch.Tensor:
@@ -140,16 +164,7 @@ def window_attention(h: torch.Tensor, st: Dict[str, torch.Tensor], p: str, m: Di
     v = v / torch.sqrt((v * v).mean(dim=-1, keepdim=True) + eps)
     window = int((m.get("mask") or {}).get("size", 0))
     sink = _w(st, p + "sink") if (p + "sink") in st else None
-    out = torch.zeros(T, H, dv, dtype=F64)
-    for i in range(T):
-        lo = max(0, i - window + 1) if window > 0 else 0
-        for hh in range(H):
-            g = hh // (H // G)
-            s = (k[lo: i + 1, g] @ q[i, hh]) * float(m["scale"])
-            mx = s.max() if sink is None else torch.maximum(s.max(), sink[hh])
-            e = torch.exp(s - mx)
-            den = e.sum() + (torch.exp(sink[hh] - mx) if sink is not None else 0.0)
-            out[i, hh] = (e / den) @ v[lo: i + 1, g]
+    out = windowed_sink_softmax(q, k, v, float(m["scale"]), window, sink)
     return out.reshape(T, H * dv) @ _w(st, p + "o").T
 
 
