@@ -676,6 +676,12 @@ def main() -> None:
                          "attention with a sink, sigmoid attention beside a state-space layer) beside the post-norm hybrid decoder of "
                          "equal size, and its kernels against their rooflines (tools/givavik_bench.py; further flags after --givavik-args)")
     ap.add_argument("--givavik-args", nargs=argparse.REMAINDER, default=[], help="flags handed to tools/givavik_bench.py")
+    ap.add_argument("--piladra", action="store_true",
+                    help="instead of the default workload: prefill / decode throughput of the looped pre-norm hybrid decoder (gated latent "
+                         "attention, selective scan, windowed attention with a sink, input-weighted experts) beside the parallel-residual "
+                         "hybrid decoder of equal size, and its kernels against their rooflines (tools/piladra_bench.py; further flags "
+                         "after --piladra-args)")
+    ap.add_argument("--piladra-args", nargs=argparse.REMAINDER, default=[], help="flags handed to tools/piladra_bench.py")
     args = ap.parse_args()
     if args.bedarax:
         from tools.bedarax_bench import main as bedarax_main
@@ -686,6 +692,11 @@ def main() -> None:
         from tools.givavik_bench import main as givavik_main
 
         givavik_main(list(args.givavik_args))
+        return
+    if args.piladra:
+        from tools.piladra_bench import main as piladra_main
+
+        piladra_main(list(args.piladra_args))
         return
     if args.hybrid:
         from tools.hybrid_bench import main as hybrid_main

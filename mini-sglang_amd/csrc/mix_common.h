@@ -69,6 +69,18 @@ __device__ __forceinline__ void read8(const bf16_t* p, float (&f)[8]) {
   f[6] = __uint_as_float(u.w << 16); f[7] = __uint_as_float(u.w & 0xffff0000u);
 }
 
+__device__ __forceinline__ void write8(float* p, const float (&f)[8]) {
+  *reinterpret_cast<float4*>(p) = float4{f[0], f[1], f[2], f[3]};
+  *reinterpret_cast<float4*>(p + 4) = float4{f[4], f[5], f[6], f[7]};
+}
+__device__ __forceinline__ void write8(bf16_t* p, const float (&f)[8]) {
+  bf16_t t[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) st(&t[i], f[i]);
+  *reinterpret_cast<uint4*>(p) = uint4{(uint32_t)t[0].bits | ((uint32_t)t[1].bits << 16), (uint32_t)t[2].bits | ((uint32_t)t[3].bits << 16),
+                                       (uint32_t)t[4].bits | ((uint32_t)t[5].bits << 16), (uint32_t)t[6].bits | ((uint32_t)t[7].bits << 16)};
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);

@@ -71,18 +71,6 @@ __global__ __launch_bounds__(256) void embed_scaled_kernel(float* __restrict__ x
 // The last token of every request leaves its h in staging[b]; commit_rows_kernel moves it to the state row after the forward
 // (a portion's first and last token run in different workgroups of this launch, so the state row cannot be replaced here).
 // A workgroup takes TT consecutive tokens; only the first of them has to rebuild the row before it.
-__device__ __forceinline__ void write8(float* p, const float (&f)[8]) {
-  *reinterpret_cast<float4*>(p) = float4{f[0], f[1], f[2], f[3]};
-  *reinterpret_cast<float4*>(p + 4) = float4{f[4], f[5], f[6], f[7]};
-}
-__device__ __forceinline__ void write8(bf16_t* p, const float (&f)[8]) {
-  bf16_t t[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) st(&t[i], f[i]);
-  *reinterpret_cast<uint4*>(p) = uint4{(uint32_t)t[0].bits | ((uint32_t)t[1].bits << 16), (uint32_t)t[2].bits | ((uint32_t)t[3].bits << 16),
-                                       (uint32_t)t[4].bits | ((uint32_t)t[5].bits << 16), (uint32_t)t[6].bits | ((uint32_t)t[7].bits << 16)};
-}
-
 // VEC: W is a multiple of 8 and every row is 16-byte aligned -- a thread takes 8 consecutive columns at a time with 16-byte loads
 // and stores; otherwise one column at a time.  Either way a thread only ever touches its own columns of the LDS rows.
 template <typename T, bool VEC>

@@ -28,6 +28,9 @@ namespace {
 __device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
 __device__ __forceinline__ float siluf_(float z) { return z / (1.0f + expf(-z)); }
 __device__ __forceinline__ float softplusf_(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+// the decay of a state element: the library's exponential in a 32-bit engine, the hardware's in a 16-bit one
+__device__ __forceinline__ float decay_exp(float z, const float*) { return expf(z); }
+__device__ __forceinline__ float decay_exp(float z, const bf16_t*) { return __expf(z); }
 
 // ------------------------------------------------------------------------------------------------ residual sum + grouped norm + input convolution
 // A workgroup owns TB consecutive new tokens of ONE request (cu_q given) or TB consecutive rows (cu_q null: no convolution over
@@ -116,16 +119,158 @@ __global__ __launch_bounds__(256) void norm_conv_kernel(const float* __restrict_
   }
 }
 
+// The same with 16-byte accesses and the ring in registers, for rows whose width and groups are multiples of 8 and at most NT <= 4 taps:
+// a thread owns NCH chunks of 8 consecutive columns (chunk j * 256 + tid), ring[NT - 1] is the current row, ring[k] the row NT - 1 - k
+// tokens before; LDS only carries the chunks' sums of squares to the waves that add up a group.
+template <typename T, int NCH, int NT>
+__global__ __launch_bounds__(256) void norm_conv_vec_kernel(const float* __restrict__ x_in, float* __restrict__ x_out, const T* __restrict__ y0,
+                                                            int p0, const T* __restrict__ y1, int p1, float mult, const float* __restrict__ add,
+                                                            const T* __restrict__ w, int groups, float eps, const T* __restrict__ taps,
+                                                            const float* __restrict__ state, float* __restrict__ staging,
+                                                            T* __restrict__ h_out, const int* __restrict__ cu_q,
+                                                            const int* __restrict__ seq_lens, const int* __restrict__ slots, int B, int rows,
+                                                            int W, int TB) {
+  extern __shared__ float lds[];
+  const int nchunks = W >> 3;
+  float* part = lds;            // [W / 8]
+  float* inv = lds + nchunks;   // [groups]
+  __shared__ int s_req, s_tok0, s_cnt[256];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int b = 0, tok_first = 0, q_len = rows, start = 0, tl0 = blockIdx.x * TB;
+  if (cu_q) {
+    find_group(cu_q, B, TB, s_cnt, &s_req, &s_tok0);
+    b = s_req;
+    if (b < 0) return;
+    tok_first = cu_q[b];
+    q_len = cu_q[b + 1] - tok_first;
+    start = seq_lens[b] - q_len;
+    tl0 = s_tok0;
+  }
+  const int cpg = (W / groups) >> 3;  // chunks per group
+  const size_t slot = cu_q && NT > 1 ? (size_t)slots[b] : 0;
+  float ring[NT][NCH][8];
+#pragma unroll
+  for (int k = 0; k < NT; ++k)
+#pragma unroll
+    for (int j = 0; j < NCH; ++j)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ring[k][j][e] = 0.f;
+  for (int i = -(NT - 1); i < TB; ++i) {
+    const int tl = tl0 + i;
+    if (tl >= q_len) break;
+#pragma unroll
+    for (int k = 0; k + 1 < NT; ++k)
+#pragma unroll
+      for (int j = 0; j < NCH; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ring[k][j][e] = ring[k + 1][j][e];
+    if (tl < 0) {  // before the portion: the request's state rows (zero before the sequence)
+      const bool have = start + tl >= 0;
+      const float* src = state + (slot * (NT - 1) + (size_t)(NT - 1 + tl)) * W;
+#pragma unroll
+      for (int j = 0; j < NCH; ++j) {
+        const int ch = j * 256 + tid;
+        if (ch < nchunks && have) {
+          read8(src + ch * 8, ring[NT - 1][j]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ring[NT - 1][j][e] = 0.f;
+        }
+      }
+      continue;
+    }
+    const size_t t = (size_t)tok_first + tl;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int ch = j * 256 + tid;
+      if (ch >= nchunks) continue;
+      const size_t c0 = (size_t)ch * 8;
+      float acc[8], v[8], s[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+      for (int p = 0; p < p0; ++p) {
+        read8(y0 + (t * p0 + p) * W + c0, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += v[e];
+      }
+      for (int p = 0; p < p1; ++p) {
+        read8(y1 + (t * p1 + p) * W + c0, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += v[e];
+      }
+      read8(x_in + t * W + c0, s);
+      if (p0 + p1 > 0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s[e] = fmaf(mult, acc[e], s[e]);
+      }
+      if (add) {
+        read8(add + c0, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s[e] += v[e];
+      }
+      if (i >= 0 && x_out) write8(x_out + t * W + c0, s);
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        ss = fmaf(s[e], s[e], ss);
+        ring[NT - 1][j][e] = s[e];
+      }
+      part[ch] = ss;
+    }
+    __syncthreads();
+    for (int g = wave; g < groups; g += 4) {
+      float ss = 0.f;
+      for (int k = lane; k < cpg; k += 64) ss += part[g * cpg + k];
+      ss = wave_sum(ss);
+      if (lane == 0) inv[g] = 1.0f / sqrtf(ss / (float)(cpg * 8) + eps);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int ch = j * 256 + tid;
+      if (ch >= nchunks) continue;
+      const size_t c0 = (size_t)ch * 8;
+      float wv[8], o[8];
+      read8(w + c0, wv);
+      const float f = inv[ch / cpg];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        ring[NT - 1][j][e] = ring[NT - 1][j][e] * f * wv[e];
+        o[e] = ring[NT - 1][j][e];
+      }
+      if (i < 0) continue;
+      if (taps) {
+        float tv[NT][8];  // the chunk's taps: element c * NT + k of 8 NT consecutive numbers
+#pragma unroll
+        for (int k = 0; k < NT; ++k) read8(taps + c0 * NT + k * 8, tv[k]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+#pragma unroll
+          for (int k = 0; k < NT; ++k) o[e] = fmaf(tv[(e * NT + k) >> 3][(e * NT + k) & 7], ring[k][j][e], o[e]);
+      }
+      write8(h_out + t * W + c0, o);
+    }
+    if (staging && NT > 1 && tl == q_len - 1) {  // the request's new state rows: the rows NT - 1 .. 1 tokens back = ring[1 ..]
+#pragma unroll
+      for (int s = 0; s + 1 < NT; ++s)
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+          const int ch = j * 256 + tid;
+          if (ch < nchunks) write8(staging + ((size_t)b * (NT - 1) + s) * W + (size_t)ch * 8, ring[s + 1][j]);
+        }
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ selective scan
 // Thread = channel c, its state row S[c, 0 : N] in NP registers (the tail unused).  Workgroup = 256 channels x (request or chunk).
 // Per token: dt = softplus(dt_in[t, c] + dt_bias[c]);  S[n] <- exp(dt A[c, n]) S[n] + dt x[t, c] B[t, n];  y = sum_n S[n] C[t, n] +
-// D[c] x[t, c];  out[t, c] = y silu(z[t, c]).  B and C of 16 tokens at a time go through LDS (every channel reads the same).
+// D[c] x[t, c];  out[t, c] = y silu(z[t, c]).  B and C of up to 16 tokens at a time go through LDS (every channel reads the same).
 // MODE 0  a request's whole portion from its state row (zero when the portion starts at position 0), state row written back.
 // Long portions are cut into chunks that run in parallel; over a chunk S_end = exp(A sum dt) S_start + L:
 // MODE 1  a chunk's L (from zero) and sum dt -> scratch, no outputs (a request's last chunk is skipped: nothing follows it);
 //         selective_join_kernel walks a request's chunks and leaves every chunk's start state where its L was;
 // MODE 2  a chunk's outputs from its start state; the last chunk of a request writes the state row.
-constexpr int kScanStage = 16;
 
 template <typename T, int NP, int MODE>
 __global__ __launch_bounds__(256) void selective_scan_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t ld_x, const T* __restrict__ z,
@@ -136,6 +281,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(T* __restrict__ out
                                                              const int* __restrict__ seq_lens, const int* __restrict__ slots, int C, int N,
                                                              const int* __restrict__ items, const int* __restrict__ item_first,
                                                              float* __restrict__ scratch, int n_items) {
+  constexpr int kScanStage = NP <= 32 ? 16 : (NP <= 64 ? 8 : 4);  // tokens staged at a time (the walk over a stage is unrolled)
   __shared__ float sB[kScanStage][NP], sC[kScanStage][NP];
   const int c = blockIdx.x * 256 + threadIdx.x;
   const bool live = c < C;
@@ -159,19 +305,38 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(T* __restrict__ out
   float S[NP], a[NP];
   float* srow = state + ((size_t)slots[b] * C + (live ? c : 0)) * N;
   float* lrow = scratch + ((size_t)it * C + (live ? c : 0)) * N;
+  const float* init = MODE == 2 ? lrow : ((MODE == 0 && !from_zero) ? srow : nullptr);
+  if (N == NP && live) {  // whole rows: 16-byte loads
 #pragma unroll
-  for (int k = 0; k < NP; ++k) {
-    a[k] = (live && k < N) ? A[(size_t)c * N + k] : 0.f;
-    S[k] = 0.f;
-    if (live && k < N) {
-      if (MODE == 0 && !from_zero) S[k] = srow[k];
-      if (MODE == 2) S[k] = lrow[k];
+    for (int k = 0; k < NP; k += 4) {
+      const float4 av = *reinterpret_cast<const float4*>(A + (size_t)c * N + k);
+      const float4 sv = init ? *reinterpret_cast<const float4*>(init + k) : float4{0.f, 0.f, 0.f, 0.f};
+      a[k] = av.x, a[k + 1] = av.y, a[k + 2] = av.z, a[k + 3] = av.w;
+      S[k] = sv.x, S[k + 1] = sv.y, S[k + 2] = sv.z, S[k + 3] = sv.w;
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < NP; ++k) {
+      a[k] = (live && k < N) ? A[(size_t)c * N + k] : 0.f;
+      S[k] = (live && k < N && init) ? init[k] : 0.f;
     }
   }
   const float bias = live ? dt_bias[c] : 0.f, skip = live ? D[c] : 0.f;
   float sumdt = 0.f;
   for (int t0 = 0; t0 < n_new; t0 += kScanStage) {
     const int nt = min(kScanStage, n_new - t0);
+    // the stage's own inputs of this channel: all loads in flight together, not one token's at a time inside the serial walk
+    float dtv[kScanStage], xv[kScanStage], zv[kScanStage];
+#pragma unroll
+    for (int tt = 0; tt < kScanStage; ++tt) {
+      dtv[tt] = xv[tt] = zv[tt] = 0.f;
+      if (tt < nt && live) {
+        const size_t t = (size_t)first + t0 + tt;
+        dtv[tt] = ld(dt_in + t * ld_dt + c);
+        xv[tt] = ld(x + t * ld_x + c);
+        if (MODE != 1) zv[tt] = ld(z + t * ld_z + c);
+      }
+    }
     __syncthreads();
     for (int e = threadIdx.x; e < nt * N; e += 256) {
       const int tt = e / N, k = e - tt * N;
@@ -181,68 +346,67 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(T* __restrict__ out
     }
     __syncthreads();
     if (!live) continue;
-    for (int tt = 0; tt < nt; ++tt) {
-      const size_t t = (size_t)first + t0 + tt;
-      const float dt = softplusf_(ld(dt_in + t * ld_dt + c) + bias);
-      const float xv = ld(x + t * ld_x + c), dx = dt * xv;
-      float y = 0.f;
 #pragma unroll
-      for (int k = 0; k < NP; ++k) {
-        if (k < N) {
-          S[k] = fmaf(expf(dt * a[k]), S[k], dx * sB[tt][k]);
-          y = fmaf(S[k], sC[tt][k], y);
+    for (int tt = 0; tt < kScanStage; ++tt) {
+      if (tt < nt) {
+        const float dt = softplusf_(dtv[tt] + bias);
+        const float dx = dt * xv[tt];
+        float y = 0.f;
+#pragma unroll
+        for (int k = 0; k < NP; ++k) {
+          if (k < N) {
+            S[k] = fmaf(decay_exp(dt * a[k], x), S[k], dx * sB[tt][k]);
+            y = fmaf(S[k], sC[tt][k], y);
+          }
         }
-      }
-      if (MODE == 1) {
-        sumdt += dt;
-      } else {
-        y = fmaf(skip, xv, y);
-        st(out + t * C + c, y * siluf_(ld(z + t * ld_z + c)));
+        if (MODE == 1) {
+          sumdt += dt;
+        } else {
+          y = fmaf(skip, xv[tt], y);
+          st(out + ((size_t)first + t0 + tt) * C + c, y * siluf_(zv[tt]));
+        }
       }
     }
   }
   if (!live) return;
-  if (MODE == 1) {
+  float* dst = MODE == 1 ? lrow : (last_chunk ? srow : nullptr);
+  if (MODE == 1) scratch[(size_t)n_items * C * N + (size_t)it * C + c] = sumdt;
+  if (!dst) return;
+  if (N == NP) {
+#pragma unroll
+    for (int k = 0; k < NP; k += 4) *reinterpret_cast<float4*>(dst + k) = float4{S[k], S[k + 1], S[k + 2], S[k + 3]};
+  } else {
 #pragma unroll
     for (int k = 0; k < NP; ++k)
-      if (k < N) lrow[k] = S[k];
-    scratch[(size_t)n_items * C * N + (size_t)it * C + c] = sumdt;
-  } else if (last_chunk) {
-#pragma unroll
-    for (int k = 0; k < NP; ++k)
-      if (k < N) srow[k] = S[k];
+      if (k < N) dst[k] = S[k];
   }
 }
 
-// Thread = (request, channel): start state of every chunk of the request, written over the chunk's L.
-template <int NP>
+// Thread = (request, one state element e = c * N + k): start state of every chunk of the request, written over the chunk's L.
 __global__ __launch_bounds__(256) void selective_join_kernel(const float* __restrict__ state, float* __restrict__ scratch,
                                                              const float* __restrict__ A, const int* __restrict__ cu_q,
                                                              const int* __restrict__ seq_lens, const int* __restrict__ slots,
                                                              const int* __restrict__ item_first, int C, int N, int n_items) {
-  const int b = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
-  if (c >= C) return;
+  const int b = blockIdx.y;
+  const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x, CN = (size_t)C * N;
+  if (e >= CN) return;
   const int i0 = item_first[b], i1 = item_first[b + 1];
   if (i1 <= i0) return;
   const bool from_zero = seq_lens[b] - (cu_q[b + 1] - cu_q[b]) == 0;
-  float S[NP], a[NP];
-#pragma unroll
-  for (int k = 0; k < NP; ++k) {
-    a[k] = k < N ? A[(size_t)c * N + k] : 0.f;
-    S[k] = (k < N && !from_zero) ? state[((size_t)slots[b] * C + c) * N + k] : 0.f;
-  }
+  const float a = A[e];
+  float S = from_zero ? 0.f : state[(size_t)slots[b] * CN + e];
+  const float* sd = scratch + (size_t)n_items * CN + e / N;
+  float L = scratch[(size_t)i0 * CN + e], d = sd[(size_t)i0 * C];
   for (int it = i0; it < i1; ++it) {
-    float* lrow = scratch + ((size_t)it * C + c) * N;
-    const float sd = scratch[(size_t)n_items * C * N + (size_t)it * C + c];
-    const bool last = it == i1 - 1;
-#pragma unroll
-    for (int k = 0; k < NP; ++k) {
-      if (k < N) {
-        const float L = lrow[k];
-        lrow[k] = S[k];
-        if (!last) S[k] = fmaf(expf(a[k] * sd), S[k], L);
-      }
+    float Ln = 0.f, dn = 0.f;
+    if (it + 1 < i1) {  // the next chunk's numbers are on their way while this one is joined
+      Ln = scratch[(size_t)(it + 1) * CN + e];
+      dn = sd[(size_t)(it + 1) * C];
     }
+    scratch[(size_t)it * CN + e] = S;
+    S = fmaf(expf(a * d), S, L);
+    L = Ln;
+    d = dn;
   }
 }
 
@@ -627,7 +791,7 @@ __global__ __launch_bounds__(256) void sigmoid_gate_kernel(T* __restrict__ out, 
 template <typename T>
 __global__ __launch_bounds__(256) void softcap_kernel(T* __restrict__ x, int64_t stride, int N, float cap, float inv_cap) {
   T* row = x + (size_t)blockIdx.x * stride;
-  for (int c = threadIdx.x; c < N; c += 256) st(row + c, cap * tanhf(ld(row + c) * inv_cap));
+  for (int c = blockIdx.y * 1024 + threadIdx.x; c < min(N, (int)(blockIdx.y + 1) * 1024); c += 256) st(row + c, cap * tanhf(ld(row + c) * inv_cap));
 }
 
 }  // namespace
@@ -644,11 +808,47 @@ int msgl_mix_norm_conv(const float* x_in, float* x_out, const void* y0, int p0, 
   MIX_REQUIRE(n == 1 || (taps && cu_q && seq_lens && slots && state && staging && batch >= 1),
               "norm_conv: a convolution over time needs taps, the requests and their state rows");
   if (rows == 0) return MSGL_MIX_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto al16 = [](const void* p) { return ((uintptr_t)p & 15u) == 0; };
+  const bool vec = W % 8 == 0 && (W / groups) % 8 == 0 && W <= 8192 && n <= 4 && al16(x_in) && al16(x_out) && al16(y0) && al16(y1) && al16(add) &&
+                   al16(w) && al16(taps) && al16(state) && al16(staging) && al16(h_out);
+  if (vec) {
+    // enough workgroups to fill the chip before a workgroup walks more tokens: a walk of TB tokens re-reads n - 1 rows
+    int TB = rows / 1024;
+    TB = TB < 1 ? 1 : (TB > 8 ? 8 : TB);
+    const int grid = cu_q ? (rows + TB - 1) / TB + batch : (rows + TB - 1) / TB;
+    const size_t lds = ((size_t)(W / 8) + groups) * sizeof(float);
+    const int nch = (W + 2047) / 2048;
+#define NC_LAUNCH(NCH, NT)                                                                                                              \
+  DISPATCH_T(dtype, hipLaunchKernelGGL((norm_conv_vec_kernel<T, NCH, NT>), dim3(grid), dim3(256), lds, s, x_in, x_out, cp<T>(y0), p0,   \
+                                       cp<T>(y1), p1, mult, add, cp<T>(w), groups, eps, cp<T>(taps), state, staging, mp<T>(h_out), cu_q, \
+                                       seq_lens, slots, batch, rows, W, TB);)
+#define NC_TAPS(NCH)       \
+  if (n == 1) {            \
+    NC_LAUNCH(NCH, 1)      \
+  } else if (n == 2) {     \
+    NC_LAUNCH(NCH, 2)      \
+  } else if (n == 3) {     \
+    NC_LAUNCH(NCH, 3)      \
+  } else {                 \
+    NC_LAUNCH(NCH, 4)      \
+  }
+    if (nch == 1) {
+      NC_TAPS(1)
+    } else if (nch == 2) {
+      NC_TAPS(2)
+    } else {
+      NC_TAPS(4)
+    }
+#undef NC_TAPS
+#undef NC_LAUNCH
+    MIX_LAUNCHED("norm_conv (16-byte accesses)");
+    return MSGL_MIX_OK;
+  }
   int TB = rows / 512;
   TB = TB < 1 ? 1 : (TB > 16 ? 16 : TB);
   const int grid = cu_q ? (rows + TB - 1) / TB + batch : (rows + TB - 1) / TB;
   const size_t lds = ((size_t)n * W + groups) * sizeof(float);
-  hipStream_t s = static_cast<hipStream_t>(stream);
   DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)norm_conv_kernel<T>, lds) == 0, "norm_conv: %d rows of %d do not fit LDS", n, W);
              hipLaunchKernelGGL(norm_conv_kernel<T>, dim3(grid), dim3(256), lds, s, x_in, x_out, cp<T>(y0), p0, cp<T>(y1), p1, mult, add,
                                 cp<T>(w), groups, eps, cp<T>(taps), n, state, staging, mp<T>(h_out), cu_q, seq_lens, slots, batch, rows, W,
@@ -680,7 +880,7 @@ int msgl_mix_selective_scan(void* out, const void* x, int64_t ld_x, const void* 
                  hipLaunchKernelGGL((selective_scan_kernel<T, NP, 1>), dim3(cb, n_items), dim3(256), 0, s, mp<T>(out), cp<T>(x), ld_x,    \
                                     cp<T>(z), ld_z, cp<T>(dt_in), ld_dt, cp<T>(bc), ld_bc, A, dt_bias, D, state, cu_q, seq_lens, slots,  \
                                     C, N, items, item_first, scratch, n_items);                                                           \
-                 hipLaunchKernelGGL(selective_join_kernel<NP>, dim3(cb, batch), dim3(256), 0, s, state, scratch, A, cu_q, seq_lens,       \
+                 hipLaunchKernelGGL(selective_join_kernel, dim3((C * N + 255) / 256, batch), dim3(256), 0, s, state, scratch, A, cu_q, seq_lens,       \
                                     slots, item_first, C, N, n_items);                                                                    \
                  hipLaunchKernelGGL((selective_scan_kernel<T, NP, 2>), dim3(cb, n_items), dim3(256), 0, s, mp<T>(out), cp<T>(x), ld_x,    \
                                     cp<T>(z), ld_z, cp<T>(dt_in), ld_dt, cp<T>(bc), ld_bc, A, dt_bias, D, state, cu_q, seq_lens, slots,  \
@@ -798,7 +998,7 @@ int msgl_mix_sigmoid_gate(void* out, const float* o, const void* g, int64_t ld_g
 int msgl_mix_softcap(void* x, int64_t ld, int rows, int N, float cap, int dtype, void* stream) {
   MIX_REQUIRE(x && dtype_ok(dtype) && rows >= 0 && N >= 1 && ld >= N && cap > 0.f, "softcap: null pointer / sizes / cap");
   if (rows == 0) return MSGL_MIX_OK;
-  DISPATCH_T(dtype, hipLaunchKernelGGL(softcap_kernel<T>, dim3(rows), dim3(256), 0, static_cast<hipStream_t>(stream), mp<T>(x), ld, N, cap,
+  DISPATCH_T(dtype, hipLaunchKernelGGL(softcap_kernel<T>, dim3(rows, (N + 1023) / 1024), dim3(256), 0, static_cast<hipStream_t>(stream), mp<T>(x), ld, N, cap,
                                        1.0f / cap);)
   MIX_LAUNCHED("softcap");
   return MSGL_MIX_OK;
