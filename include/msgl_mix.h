@@ -266,6 +266,11 @@ int msgl_mix_route_sigmoid(int* ids, float* wts, const float* z, int tokens, int
 /* out[t * top + k, :] = wts[t, k] * h[t, :] (T rows of W): the inputs of experts that are weighted before they run. */
 int msgl_mix_scale_rows(void* out, const void* h, const float* wts, int tokens, int top, int W, int dtype, void* stream);
 
+/* The three steps above in one launch, a workgroup per token (for steps with few tokens): z = router h (router T [E, W], fp32
+ * accumulation), the `top` largest, out[t * top + k, :] = sigmoid(z of choice k) * h[t, :]; ids, wts as above. */
+int msgl_mix_route_scale(int* ids, float* wts, void* out, const void* h, const void* router, int tokens, int E, int top, int W, int dtype,
+                         void* stream);
+
 /* out (T [rows, N]) = o (fp32 [rows, N]) * sigmoid(g) (T rows ld_g apart). */
 int msgl_mix_sigmoid_gate(void* out, const float* o, const void* g, int64_t ld_g, int rows, int N, int dtype, void* stream);
 

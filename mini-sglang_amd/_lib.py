@@ -179,6 +179,7 @@ MIX_SIGNATURES = {
     "msgl_mix_sink_attn": (_i, [_p, _l, _p, _p, _p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _p, _i, _i, _p, _p]),
     "msgl_mix_route_sigmoid": (_i, [_p, _p, _p, _i, _i, _i, _p]),
     "msgl_mix_scale_rows": (_i, [_p, _p, _p, _i, _i, _i, _i, _p]),
+    "msgl_mix_route_scale": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
     "msgl_mix_sigmoid_gate": (_i, [_p, _p, _p, _l, _i, _i, _i, _p]),
     "msgl_mix_softcap": (_i, [_p, _l, _i, _i, _f, _i, _p]),
 }

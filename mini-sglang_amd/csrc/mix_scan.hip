@@ -19,6 +19,7 @@
 //   sink_attn_kernel        the same in plain fp32 (fp32 caches, heads past the matrix-core instances)
 //   route_sigmoid_kernel    the `top` largest router logits win, weights = sigmoid(logit)
 //   scale_rows_kernel       one copy of a token's row per chosen expert, multiplied by that choice's weight
+//   route_scale_kernel      logits, choice and scaled rows of a token in one launch (steps with few tokens)
 //   sigmoid_gate_kernel     out = o * sigmoid(g)
 //   softcap_kernel          x <- cap tanh(x / cap)
 #include "mix_common.h"
@@ -781,6 +782,59 @@ __global__ __launch_bounds__(256) void scale_rows_kernel(T* __restrict__ out, co
   for (int c = threadIdx.x; c < W; c += 256) st(out + r * W + c, f * ld(src + c));
 }
 
+// Router logits, choice and the scaled rows of ONE token per workgroup, for steps with few tokens (every token re-reads the router
+// matrix, so long batches take the product kernel for the logits instead): z[e] = router[e] . h (fp32 accumulation over the row as
+// stored), the `top` largest win, out[t * top + k] = sigmoid(z[best_k]) * h[t].
+template <typename T>
+__global__ __launch_bounds__(256) void route_scale_kernel(int* __restrict__ ids, float* __restrict__ wts, T* __restrict__ out,
+                                                          const T* __restrict__ h, const T* __restrict__ router, int E, int top, int W) {
+  extern __shared__ float lds[];
+  float* row = lds;       // [W]
+  float* z = lds + W;     // [E]
+  float* sel = z + E;     // [top]
+  const size_t t = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int c = tid; c < W; c += 256) row[c] = ld(h + t * W + c);
+  __syncthreads();
+  const bool vec = (W & 7) == 0 && ((uintptr_t)router & 15u) == 0;
+  for (int e = wave; e < E; e += 4) {
+    const T* r = router + (size_t)e * W;
+    float acc = 0.f;
+    if (vec) {  // 16-byte loads of the expert's row, several in flight
+      for (int c0 = lane * 8; c0 < W; c0 += 512) {
+        float wv[8];
+        read8(r + c0, wv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc = fmaf(row[c0 + i], wv[i], acc);
+      }
+    } else {
+      for (int c = lane; c < W; c += 64) acc = fmaf(row[c], ld(r + c), acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) z[e] = acc;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    for (int k = 0; k < top; ++k) {
+      int best = 0;
+      float bv = -INFINITY;
+      for (int e = 0; e < E; ++e)
+        if (z[e] > bv) {
+          best = e;
+          bv = z[e];
+        }
+      ids[t * top + k] = best;
+      sel[k] = wts[t * top + k] = sigmoidf_(bv);
+      z[best] = -INFINITY;
+    }
+  }
+  __syncthreads();
+  for (int k = 0; k < top; ++k) {
+    const float f = sel[k];
+    for (int c = tid; c < W; c += 256) st(out + (t * top + k) * W + c, f * row[c]);
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void sigmoid_gate_kernel(T* __restrict__ out, const float* __restrict__ o, const T* __restrict__ g,
                                                            int64_t ld_g, int N) {
@@ -983,6 +1037,19 @@ int msgl_mix_scale_rows(void* out, const void* h, const float* wts, int tokens, 
   DISPATCH_T(dtype, hipLaunchKernelGGL(scale_rows_kernel<T>, dim3(tokens * top), dim3(256), 0, static_cast<hipStream_t>(stream), mp<T>(out),
                                        cp<T>(h), wts, top, W);)
   MIX_LAUNCHED("scale_rows");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_route_scale(int* ids, float* wts, void* out, const void* h, const void* router, int tokens, int E, int top, int W, int dtype,
+                         void* stream) {
+  MIX_REQUIRE(ids && wts && out && h && router && dtype_ok(dtype), "route_scale: null pointer / dtype");
+  MIX_REQUIRE(tokens >= 0 && E >= 1 && top >= 1 && top <= E && W >= 1, "route_scale: bad sizes E %d top %d", E, top);
+  if (tokens == 0) return MSGL_MIX_OK;
+  const size_t lds = ((size_t)W + E + top) * sizeof(float);
+  DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)route_scale_kernel<T>, lds) == 0, "route_scale: a row of %d and %d experts do not fit LDS", W, E);
+             hipLaunchKernelGGL(route_scale_kernel<T>, dim3(tokens), dim3(256), lds, static_cast<hipStream_t>(stream), ids, wts, mp<T>(out),
+                                cp<T>(h), cp<T>(router), E, top, W);)
+  MIX_LAUNCHED("route_scale");
   return MSGL_MIX_OK;
 }
 

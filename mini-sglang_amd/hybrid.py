@@ -917,8 +917,13 @@ class HybridDecoder:
         """-> [T, top, W]: every chosen expert's output on score * h (the score is inside the expert's input, so the caller adds the
         rows as they are)."""
         m, (T, W) = L.spec.mlp, h.shape
-        ids, wts = mixops.route_sigmoid(h, L.router, m.top)
-        hs = mixops.scale_rows(h, wts)
+        # few tokens (decode, short portions): logits, choice and the scaled rows leave one launch; many tokens: every token re-reading
+        # the router matrix costs more than the launches it saves, so the logits come from the product kernel
+        if T <= self.ROUTE_FUSE_MAX_TOKENS:
+            ids, _, hs = mixops.route_scale(h, L.router, m.top)
+        else:
+            ids, wts = mixops.route_sigmoid(h, L.router, m.top)
+            hs = mixops.scale_rows(h, wts)
         seg, perm = mixops.moe_sort(ids, m.experts)
         n = T * m.top
         gu = torch.empty((n, 2 * m.ff), dtype=self.dtype, device=h.device)

@@ -740,6 +740,20 @@ def scale_rows(h: torch.Tensor, wts: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def route_scale(h: torch.Tensor, router: torch.Tensor, top: int):
+    """route_sigmoid and scale_rows in one launch, a workgroup per token (steps with few tokens) -> (ids, weights, scaled rows)."""
+    _dev(h, router)
+    T, W = h.shape
+    E = router.shape[0]
+    assert h.is_contiguous() and router.is_contiguous() and router.shape == (E, W) and router.dtype == h.dtype
+    ids = torch.empty((T, top), dtype=torch.int32, device=h.device)
+    wts = torch.empty((T, top), dtype=torch.float32, device=h.device)
+    out = torch.empty((T * top, W), dtype=h.dtype, device=h.device)
+    check_mix(mix_lib().msgl_mix_route_scale(ids.data_ptr(), wts.data_ptr(), out.data_ptr(), h.data_ptr(), router.data_ptr(), T, E, top, W,
+                                             _code(h), _stream()), "route_scale")
+    return ids, wts, out
+
+
 def sigmoid_gate(o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
     """-> o * sigmoid(g) in g's dtype; o fp32 [rows, N], g a [rows, N] view with a row stride."""
     _dev(o, g)
