@@ -310,6 +310,32 @@ def test_window_attention_sinks_and_batches(dev, dtype):
         assert float(got[:, 0].abs().max()) < 1e-2 * float(got[:, 1].abs().max())
 
 
+@pytest.mark.parametrize("H,G,d,dv", [(4, 4, 32, 32), (8, 2, 64, 64), (6, 3, 48, 40), (3, 1, 96, 80), (16, 2, 128, 128), (2, 1, 192, 104), (8, 1, 256, 256),
+                                      (5, 5, 72, 136)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_window_attention_head_sizes(dev, dtype, H, G, d, dv):
+    """Every matrix-core instance (and the plain kernel beside it): head sizes from 32 to 256, one to eight query heads per key head,
+    a window that ends inside a tile, a portion after a cached prefix and single tokens, keys in one range and in two."""
+    from mini_sglang_amd import mixops
+
+    T, window, scale = 150, 45, d ** -0.5
+    g = torch.Generator().manual_seed(d + dv)
+    q, k, v = (torch.randn(T, n, w, generator=g, dtype=torch.float64).to(dtype).double() for n, w in ((H, d), (G, d), (G, dv)))
+    sink = torch.randn(H, generator=g, dtype=torch.float64)
+    ref = O.windowed_sink_softmax(q, k, v, scale, window, sink)
+    table, kc, vc = _paged(dev, T, k, v, dtype, g)
+    qd = q.reshape(T, -1).float().to(dev)
+    for splits in (1, 2):
+        got = torch.empty((T, H * dv), dtype=dtype, device=dev)
+        for lo, hi in _pieces(T, 70, 30):
+            part = torch.empty((hi - lo, H * dv), dtype=dtype, device=dev)
+            mixops.sink_attn(part, qd[lo:hi].contiguous(), kc, vc, table, torch.tensor([2], dtype=torch.int32, device=dev),
+                             torch.tensor([hi], dtype=torch.int32, device=dev), torch.tensor([0, hi - lo], dtype=torch.int32, device=dev),
+                             1, H, G, d, dv, scale, window, sink.float().to(dev), splits=splits)
+            got[lo:hi] = part
+        assert rel(got.double().cpu().view(T, H, dv), ref) < (1e-5 if dtype == torch.float32 else 2e-2), splits
+
+
 @pytest.mark.parametrize("chunk", [0, 1, 5], ids=["whole", "chunks-of-1", "chunks-of-5"])
 def test_selective_scan_kernel_state_slots_and_cuts(dev, chunk):
     """The recurrence kernel alone: two requests in one launch on state rows that hold garbage, then continued in a second
@@ -472,6 +498,19 @@ def test_other_orders_and_sizes_bf16():
     a, b = tokens_of(140, 200, 61), tokens_of(33, 200, 62)
     steps = [[("a", a[:100], False)], [("a", a[100:101], False), ("b", b[:20], False)], [("a", a[101:], True), ("b", b[20:], True)]]
     check(engine_for(cfg, torch.bfloat16), cfg, steps, {"a": a, "b": b}, BF16_TOL, allow=0.05)
+
+
+def test_wider_model_with_odd_head_sizes_bf16():
+    """Head sizes, ranks and channel counts that are no powers of two, three key heads, two input taps, three norm groups, a run of two
+    layers three times; two requests whose portions and single tokens share steps."""
+    cfg = config([att(heads=6, kv_heads=3, dim=48, vdim=40, dims=24, window=33, mlp=moe(experts=5, top=3, ff=40, shared=24)),
+                  mam(inner=384, state=8, dt_rank=6, conv=2, mlp=dense(ff=200)),
+                  lat(heads=3, dim=48, rot_dim=32, vdim=56, kv_rank=80, mlp=None)], width=192, vocab=333, groups=3, taps=2, loop=(0, 2, 3))
+    a, b = tokens_of(120, 333, 63), tokens_of(70, 333, 64)
+    steps = [[("a", a[:64], False)], [("a", a[64:65], False), ("b", b[:50], False)], [("a", a[65:66], False), ("b", b[50:51], False)],
+             [("a", a[66:], True), ("b", b[51:], True)]]
+    check(engine_for(cfg, torch.bfloat16), cfg, steps, {"a": a, "b": b}, BF16_TOL, allow=0.05)
+    check(engine_for(cfg, torch.float32), cfg, steps, {"a": a, "b": b}, FP32_TOL)
 
 
 @pytest.mark.parametrize("graphs", [None, [1, 2, 4]], ids=["eager", "graphs"])
