@@ -32,6 +32,13 @@ __device__ __forceinline__ float softplusf_(float z) { return z > 20.0f ? z : lo
 // the decay of a state element: the library's exponential in a 32-bit engine, the hardware's in a 16-bit one
 __device__ __forceinline__ float decay_exp(float z, const float*) { return expf(z); }
 __device__ __forceinline__ float decay_exp(float z, const bf16_t*) { return __expf(z); }
+// the same split for the scan's step size and gate (once per token and channel, but inside the serial walk)
+__device__ __forceinline__ float scan_softplus(float z, const float*) { return softplusf_(z); }
+__device__ __forceinline__ float scan_softplus(float z, const bf16_t*) {
+  return z > 20.0f ? z : (z < -15.0f ? __expf(z) : __logf(1.0f + __expf(z)));
+}
+__device__ __forceinline__ float scan_silu(float z, const float*) { return siluf_(z); }
+__device__ __forceinline__ float scan_silu(float z, const bf16_t*) { return z * __builtin_amdgcn_rcpf(1.0f + __expf(-z)); }
 
 // ------------------------------------------------------------------------------------------------ residual sum + grouped norm + input convolution
 // A workgroup owns TB consecutive new tokens of ONE request (cu_q given) or TB consecutive rows (cu_q null: no convolution over
@@ -350,7 +357,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(T* __restrict__ out
 #pragma unroll
     for (int tt = 0; tt < kScanStage; ++tt) {
       if (tt < nt) {
-        const float dt = softplusf_(dtv[tt] + bias);
+        const float dt = scan_softplus(dtv[tt] + bias, x);
         const float dx = dt * xv[tt];
         float y = 0.f;
 #pragma unroll
@@ -364,7 +371,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(T* __restrict__ out
           sumdt += dt;
         } else {
           y = fmaf(skip, xv[tt], y);
-          st(out + ((size_t)first + t0 + tt) * C + c, y * siluf_(zv[tt]));
+          st(out + ((size_t)first + t0 + tt) * C + c, y * scan_silu(zv[tt], x));
         }
       }
     }
